@@ -5,7 +5,9 @@
 //     gla:    g = sigmoid(a + a_bias)^(1/tau);              S <- g S + k v^T;            o = S^T q
 //     delta:  g = exp(-exp(A_log[h]) softplus(a + a_bias));  S <- g S;  u = b (v - S^T k);
 //             S <- S + k u^T;  o = S^T q;    q, k unit vectors per head first, b = sigmoid(beta)
-//   and q scaled by D^-1/2 in both.  Two launches:
+//   and q scaled by D^-1/2 in both; or (mx_decay_scan) one FIXED decay per head,
+//     fixed:  S <- decay[h] S + act(k) act(v)^T;  o = S^T act(q) * out_scale
+//   with the activation (none | SiLU) applied while the rows are staged and no prep launch.  Two launches:
 //     prep   one block per token, fully parallel: the decays g (written over `a`), and for the delta
 //            rule the unit-norm factors of q and k and sigmoid(beta) (steps of single rows -- decode --
 //            skip this launch: the scan's one-token form computes them while it stages the row);
@@ -73,7 +75,9 @@ __global__ void scan_prep_kernel(const TQ* __restrict__ q, long sq, const TQ* __
 }
 
 // grid (ceil(P / CB), H, S), 256 threads = CB columns x LPC lanes, CB = 256 / LPC
-template <typename TQ, int RPL, int LPC, bool DELTA, bool ONE>      // ONE: every segment is a single row (decode)
+// MODE 0: gla, 1: delta, 2: fixed decay per head (a_bias = decay [H], tau_inv = the output scale, beta_code =
+// activation code | storage code of v << 4; q and k of type TQ, no g / aux / beta)
+template <typename TQ, int RPL, int LPC, int MODE, bool ONE>      // ONE: every segment is a single row (decode)
 __global__ void __launch_bounds__(256)
 matrix_scan_kernel(const TQ* __restrict__ q, long sq, const TQ* __restrict__ k, long sk, const TQ* __restrict__ v, long sv,
                    const float* __restrict__ gdec, long sa, const float* __restrict__ aux, float* __restrict__ state,
@@ -81,6 +85,7 @@ matrix_scan_kernel(const TQ* __restrict__ q, long sq, const TQ* __restrict__ k, 
                    float* __restrict__ out, int H, int G, int D, int P, const float* __restrict__ a_bias,
                    const float* __restrict__ A_log, const void* __restrict__ beta, long sbeta, int beta_code,
                    float tau_inv) {
+  constexpr bool DELTA = MODE == 1, FIXED = MODE == 2;
   constexpr int DP = RPL * LPC;          // padded key size
   constexpr int CB = 256 / LPC;          // columns per block
   constexpr int TB = ONE ? 1 : (DP <= 256 ? 16 : 8);   // tokens per chunk
@@ -88,7 +93,7 @@ matrix_scan_kernel(const TQ* __restrict__ q, long sq, const TQ* __restrict__ k, 
   constexpr int NV = (TB * CB + 255) / 256;
   __shared__ __align__(16) float qs[TB * DP];
   __shared__ __align__(16) float ks[TB * DP];
-  __shared__ __align__(16) float gs[TB * DP];
+  __shared__ __align__(16) float gs[FIXED ? 4 : TB * DP];
   __shared__ float vs[TB * CB];
   __shared__ float os[TB * CB];
   __shared__ float bs[TB];
@@ -103,6 +108,8 @@ matrix_scan_kernel(const TQ* __restrict__ q, long sq, const TQ* __restrict__ k, 
   const bool fresh = pos[r0] == 0;
   const float qscale = 1.0f / sqrtf((float)D);
   const int AW = 2 * G + H;              // aux row width
+  const float gfix = FIXED ? a_bias[h] : 1.f;
+  const int fact = beta_code & 15, vcode = beta_code >> 4;
 
   float S[RPL];
   float* srec = state + (((long)sl * H + h) * D) * P;
@@ -122,7 +129,14 @@ matrix_scan_kernel(const TQ* __restrict__ q, long sq, const TQ* __restrict__ k, 
       const int t = e / DP, d = e - t * DP;
       const long row = r0 + min(t0 + t, n - 1);
       const int dc = min(d, D - 1);
-      if (ONE) {       // no prep pass ran: the decay from its pre-activation here, the unit norms after staging
+      if (FIXED) {
+        pq[i] = ldf(q + row * sq + kvh * D + dc);
+        pk[i] = ldf(k + row * sk + kvh * D + dc);
+        if (fact == 1) {
+          pq[i] = mx_silu(pq[i]);
+          pk[i] = mx_silu(pk[i]);
+        }
+      } else if (ONE) {       // no prep pass ran: the decay from its pre-activation here, the unit norms after staging
         pq[i] = ldf(q + row * sq + kvh * D + dc);
         pk[i] = ldf(k + row * sk + kvh * D + dc);
         const float z = gdec[row * sa + h * D + dc] + a_bias[h * D + dc];
@@ -138,7 +152,13 @@ matrix_scan_kernel(const TQ* __restrict__ q, long sq, const TQ* __restrict__ k, 
     for (int i = 0; i < NV; ++i) {
       const int e = min(tid + 256 * i, TB * CB - 1);
       const int t = e / CB, c = e - t * CB;
-      pv[i] = ldf(v + (long)(r0 + min(t0 + t, n - 1)) * sv + h * P + min(c0 + c, P - 1));
+      const long vi = (long)(r0 + min(t0 + t, n - 1)) * sv + h * P + min(c0 + c, P - 1);
+      if (FIXED) {
+        pv[i] = ld_code(v, vcode, vi);
+        if (fact == 1) pv[i] = mx_silu(pv[i]);
+      } else {
+        pv[i] = ldf(v + vi);
+      }
     }
     if (DELTA && tid < TB)
       pb = ONE ? mx_sigmoid(ld_code(beta, beta_code, (long)(r0 + min(t0 + tid, n - 1)) * sbeta + h))
@@ -155,7 +175,7 @@ matrix_scan_kernel(const TQ* __restrict__ q, long sq, const TQ* __restrict__ k, 
         const bool live = (e % DP) < D;
         qs[e] = live ? pq[i] : 0.f;
         ks[e] = live ? pk[i] : 0.f;
-        gs[e] = live ? pg[i] : 1.f;
+        if (!FIXED) gs[e] = live ? pg[i] : 1.f;
       }
     }
 #pragma unroll
@@ -206,7 +226,9 @@ matrix_scan_kernel(const TQ* __restrict__ q, long sq, const TQ* __restrict__ k, 
 #pragma unroll
       for (int i4 = 0; i4 < RPL / 4; ++i4) {
         const float4 qq = qr[i4];
-        if (!DELTA) {
+        if (FIXED) {
+          S[4 * i4] *= gfix; S[4 * i4 + 1] *= gfix; S[4 * i4 + 2] *= gfix; S[4 * i4 + 3] *= gfix;
+        } else if (!DELTA) {
           const float4 gg = gr[i4];
           S[4 * i4] *= gg.x; S[4 * i4 + 1] *= gg.y; S[4 * i4 + 2] *= gg.z; S[4 * i4 + 3] *= gg.w;
         }
@@ -217,7 +239,7 @@ matrix_scan_kernel(const TQ* __restrict__ q, long sq, const TQ* __restrict__ k, 
         o += S[4 * i4] * qq.x + S[4 * i4 + 1] * qq.y + S[4 * i4 + 2] * qq.z + S[4 * i4 + 3] * qq.w;
       }
       o = lane_group_sum<LPC>(o);
-      if (part == 0) os[t * CB + cl] = DELTA ? o : o * qscale;     // delta: the scale is part of q's norm factor
+      if (part == 0) os[t * CB + cl] = DELTA ? o : o * (FIXED ? tau_inv : qscale);   // delta: the scale is part of q's norm factor
     }
     __syncthreads();
     for (int e = tid; e < nt * CB; e += 256) {
@@ -344,7 +366,7 @@ __global__ void lru_step_kernel(const float* __restrict__ u, const float* __rest
   }
 }
 
-template <typename TQ, int RPL, int LPC, bool DELTA>
+template <typename TQ, int RPL, int LPC, int DELTA>
 int launch_matrix_scan(const void* q, long sq, const void* k, long sk, const void* v, long sv, const float* g, long sa,
                        const float* aux, float* state, const int* cu, const int* slot, const int* pos, float* out, int S,
                        int H, int G, int D, int P, const float* a_bias, const float* A_log, const void* beta, long sbeta,
@@ -363,7 +385,7 @@ int launch_matrix_scan(const void* q, long sq, const void* k, long sk, const voi
 }
 
 // the variant with 16 lanes per column when the narrow one would leave most of the chip idle
-template <typename TQ, bool DELTA, typename... Args>
+template <typename TQ, int DELTA, typename... Args>
 int dispatch_matrix_scan(int D, bool wide, Args... args) {
   if (D <= 32) return launch_matrix_scan<TQ, 8, 4, DELTA>(args...);
   if (D <= 64) return wide ? launch_matrix_scan<TQ, 4, 16, DELTA>(args...) : launch_matrix_scan<TQ, 16, 4, DELTA>(args...);
@@ -418,6 +440,30 @@ MX_API int mx_matrix_scan(const void* q, long sq, const void* k, long sk, const 
                                          cu, slot, pos, out, S, T, H, G, D, P, max_len, st);
   return run_matrix_scan<bf16, false>(q, sq, k, sk, v, sv, a, sa, a_bias, A_log, beta, sbeta, beta_dt, ti, aux, state, cu,
                                       slot, pos, out, S, T, H, G, D, P, max_len, st);
+}
+
+// One fixed decay per head: S <- decay[h] S + act(k) act(v)^T, o = S^T act(q) * out_scale.  q, k [rows, H*D]
+// slices of storage type dt_qk, v [rows, H*P] slice of type dt_v (the two may differ: rotated f32 q, k beside
+// the projection's own v); act 0: none, 1: SiLU on q, k and v; decay f32 [H]; state f32 [slots, H, D, P];
+// out f32 [T, H*P].  One launch, also for prompt chunks.
+MX_API int mx_decay_scan(const void* q, long sq, const void* k, long sk, int dt_qk, const void* v, long sv, int dt_v,
+                         int act, const float* decay, float out_scale, float* state, const int* cu, const int* slot,
+                         const int* pos, float* out, int S, int T, int max_len, int H, int D, int P, hipStream_t st) {
+  if (S <= 0 || T <= 0) return 0;
+  if (D < 1 || D > 512 || decay == nullptr || (act != 0 && act != 1)) return (int)hipErrorInvalidValue;
+  const bool one = max_len == 1;
+  const long seff = max_len > 0 ? (S < (T + max_len - 1) / max_len ? S : (T + max_len - 1) / max_len) : S;
+  const int lpc = D <= 128 ? 4 : (D <= 256 ? 8 : 16);
+  const long blocks = seff * H * ((P + 256 / lpc - 1) / (256 / lpc));
+  const int code = act | (dt_v << 4);
+  // v travels as an untyped pointer: the fixed mode reads it by its storage code
+  if (dt_qk == 1)
+    return dispatch_matrix_scan<float, 2>(D, blocks < 512, q, sq, k, sk, v, sv, (const float*)nullptr, 0L,
+                                          (const float*)nullptr, state, cu, slot, pos, out, S, H, H, D, P, decay,
+                                          (const float*)nullptr, (const void*)nullptr, 0L, code, out_scale, one, st);
+  return dispatch_matrix_scan<bf16, 2>(D, blocks < 512, q, sq, k, sk, v, sv, (const float*)nullptr, 0L,
+                                       (const float*)nullptr, state, cu, slot, pos, out, S, H, H, D, P, decay,
+                                       (const float*)nullptr, (const void*)nullptr, 0L, code, out_scale, one, st);
 }
 
 // u f32 [T, R], OVERWRITTEN with the GeLU branch; z f32 [blocks, T, 2 * R / blocks], OVERWRITTEN with the gates; y [T, >= R] slice (row stride

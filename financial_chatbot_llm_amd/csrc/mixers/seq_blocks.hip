@@ -122,7 +122,8 @@ __global__ void glu_act_kernel(const T* __restrict__ gate, long sg, const T* __r
 }
 
 // one wave per token: the `top` largest scores (ties: the lower index) with the score as weight.
-// sigmoid scores keep the order of the logits; softmax scores are normalised over all E entries.
+// sigmoid scores (1) keep the order of the logits; softmax scores are normalised over all E entries (0)
+// or over the chosen entries only (2).
 __global__ void route_scores_kernel(const float* __restrict__ z, int E, int top, int sigmoid_scores,
                                     float* __restrict__ outw, int* __restrict__ outi, int T) {
   const int t = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
@@ -130,7 +131,7 @@ __global__ void route_scores_kernel(const float* __restrict__ z, int E, int top,
   if (t >= T) return;
   const float* zr = z + (long)t * E;
   float m = -INFINITY, inv = 1.f;
-  if (!sigmoid_scores) {
+  if (sigmoid_scores == 0) {
     for (int e = lane; e < E; e += 64) m = fmaxf(m, zr[e]);
     m = mx_wave_max(m);
     float s = 0.f;
@@ -166,12 +167,24 @@ __global__ void route_scores_kernel(const float* __restrict__ z, int E, int top,
     if (lane == 0) {
       const int e = bi == 0x7fffffff ? 0 : bi;
       outi[(long)t * top + k] = e;
-      outw[(long)t * top + k] = bi == 0x7fffffff ? 0.f : (sigmoid_scores ? mx_sigmoid(zr[e]) : expf(zr[e] - m) * inv);
+      outw[(long)t * top + k] = bi == 0x7fffffff ? 0.f : (sigmoid_scores == 1 ? mx_sigmoid(zr[e])
+                                : sigmoid_scores == 2 ? zr[e] : expf(zr[e] - m) * inv);
     }
+  }
+  if (sigmoid_scores == 2 && lane == 0) {       // softmax over the chosen logits (the first is the largest)
+    float* w = outw + (long)t * top;
+    const float m2 = w[0];
+    float s = 0.f;
+    for (int k = 0; k < top; ++k) {
+      w[k] = expf(w[k] - m2);
+      s += w[k];
+    }
+    const float r = 1.0f / s;
+    for (int k = 0; k < top; ++k) w[k] *= r;
   }
 }
 
-// grid (rows, H): head h's P outputs / rms * w[P] * act(gate)
+// grid (rows, H): head h's P outputs / rms * w[P] * act(gate); w null: no weight
 template <typename TI, typename TG, typename TO>
 __global__ void head_norm_gate_kernel(const TI* __restrict__ in, long si, const float* __restrict__ w, float eps,
                                       const TG* __restrict__ gate, long sg, int act, TO* __restrict__ out, int P) {
@@ -187,7 +200,8 @@ __global__ void head_norm_gate_kernel(const TI* __restrict__ in, long si, const 
   ss = mx_block_sum(ss, scratch);
   const float k = 1.0f / sqrtf(ss / (float)P + eps);
   for (int i = threadIdx.x; i < P; i += blockDim.x)
-    stf(out + (t * H + h) * P + i, ldf(r + i) * k * w[i] * mx_act(ldf(gate + t * sg + (long)h * P + i), act));
+    stf(out + (t * H + h) * P + i,
+        ldf(r + i) * k * (w != nullptr ? w[i] : 1.f) * mx_act(ldf(gate + t * sg + (long)h * P + i), act));
 }
 
 }  // namespace
@@ -236,7 +250,7 @@ MX_API int mx_route_scores(const float* z, int E, int top, int sigmoid_scores, f
 }
 
 // in [T, H*P] (row stride si, type dt_in), gate [T, H*P] slice (row stride sg, type dt_gate), out [T, H*P]
-// contiguous of type dt_out; act: 1 SiLU, 3 sigmoid
+// contiguous of type dt_out; w f32 [P] or null; act: 1 SiLU, 3 sigmoid
 MX_API int mx_head_norm_gate(const void* in, long si, int dt_in, const float* w, float eps, const void* gate, long sg,
                              int dt_gate, int act, void* out, int dt_out, int T, int H, int P, hipStream_t st) {
   if (T <= 0) return 0;

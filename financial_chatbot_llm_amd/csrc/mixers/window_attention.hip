@@ -2,8 +2,11 @@
 //
 // The cache row of a token is [k: G*D | v: G*P] (G key/value heads of key size D and value size P).
 // Query head h reads key/value head h / (H / G).  The query at position p sees the keys j of its own
-// sequence with 0 <= p - j < window; score = q . k * scale; softmax and accumulation in f32; the
-// head's output is multiplied by sigmoid(gate[t, h]) when a gate is given.  No positional rotation.
+// sequence with 0 <= p - j < window -- or, chunked, the keys j <= p of its own block of `window`
+// positions (floor(j / window) == floor(p / window), blocks counted from position 0 of the sequence);
+// score = q . k * scale; softmax and accumulation in f32; the head's output is multiplied by
+// sigmoid(gate[t, h]) when a gate is given.  Rotation and norms of q and k happen before (the cache holds
+// finished keys).
 //
 //   mx_qk_norm_write   RMS norm over the WHOLE query projection and over the whole key projection
 //                      (all heads at once, plain weights), cache write of [normed k | v].
@@ -16,6 +19,11 @@
 namespace {
 
 constexpr int PAGE = 64;            // tokens per cache page
+
+// first key the query at position p sees: a sliding window of `window` keys, or the start of p's block
+__device__ __forceinline__ int first_key(int p, int window, int chunked) {
+  return chunked ? (p / window) * window : max(0, p - window + 1);
+}
 
 // one block per token
 template <typename T>
@@ -66,8 +74,8 @@ template <typename T>
 __global__ void __launch_bounds__(WA_WAVES * 64)
 window_attend_kernel(const T* __restrict__ q, long sq, const T* __restrict__ cache, const int* __restrict__ cu,
                      const int* __restrict__ pos, const int* __restrict__ bt, int btw, const T* __restrict__ gate,
-                     long sgate, int window, float scale, T* __restrict__ out, int H, int G, int D, int P, int QT,
-                     int HB, int KT, int ldk, int ldv) {
+                     long sgate, int window, int chunked, float scale, T* __restrict__ out, int H, int G, int D, int P,
+                     int QT, int HB, int KT, int ldk, int ldv) {
   extern __shared__ __align__(16) unsigned char smem[];
   T* ktile = reinterpret_cast<T*>(smem);                                  // [KT][ldk]
   T* vtile = ktile + (size_t)KT * ldk;                                    // [KT][ldv]
@@ -86,7 +94,7 @@ window_attend_kernel(const T* __restrict__ q, long sq, const T* __restrict__ cac
   const int h0 = g * rep + hg0;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int p_first = pos[r0 + t0], p_last = pos[r0 + t0 + nq - 1];
-  const int lo = max(0, p_first - window + 1);
+  const int lo = first_key(p_first, window, chunked);
   const int nitems = nq * nh;
   const int Wr = G * (D + P);
   const int koff = g * D, voff = G * D + g * P;
@@ -126,7 +134,7 @@ window_attend_kernel(const T* __restrict__ q, long sq, const T* __restrict__ cac
       const int h = h0 + hh;
       const int p = pos[row];
       const int j = k0 + lane;
-      const bool vis = lane < rows && j <= p && j > p - window;
+      const bool vis = lane < rows && j <= p && j >= first_key(p, window, chunked);
       if (__ballot(vis) == 0ull) continue;                // no visible key of this tile
       {
         const T* qh = q + row * sq + (long)h * D;
@@ -201,8 +209,9 @@ template <int KSM, int NTM>         // up to 32*KSM key dims, 16*NTM value dims
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
 window_attend_mfma_kernel(const bf16* __restrict__ q, long sq, const bf16* __restrict__ cache,
                           const int* __restrict__ cu, const int* __restrict__ pos, const int* __restrict__ bt, int btw,
-                          const bf16* __restrict__ gate, long sgate, int window, float scale, bf16* __restrict__ out,
-                          int H, int G, int D, int P, int QT, int HB, int nsplit, float* __restrict__ ws) {
+                          const bf16* __restrict__ gate, long sgate, int window, int chunked, float scale,
+                          bf16* __restrict__ out, int H, int G, int D, int P, int QT, int HB, int nsplit,
+                          float* __restrict__ ws) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int KS = (D + 31) / 32, NT = (P + 15) / 16;
   const int ldk = KS * 32 + 8;
@@ -225,7 +234,7 @@ window_attend_mfma_kernel(const bf16* __restrict__ q, long sq, const bf16* __res
   const int koff = kvh * D, voff = G * D + kvh * P;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 4, c = lane & 15;
   const int p_first = pos[r0 + t0], p_last = pos[r0 + t0 + nq - 1];
-  const int lo = max(0, p_first - window + 1);
+  const int lo = first_key(p_first, window, chunked);
   // this lane's query: pair index 16 * wave + c
   const int pair = 16 * wave + c;
   const bool qok = pair < nq * nh;
@@ -233,6 +242,7 @@ window_attend_mfma_kernel(const bf16* __restrict__ q, long sq, const bf16* __res
   const long row = r0 + t0 + tq;
   const int h = h0 + hh;
   const int pq = qok ? pos[row] : -1;
+  const int pq_lo = qok ? first_key(pq, window, chunked) : 0;
   const bool wave_live = 16 * wave < nq * nh;
 
   bf16x8 qf[KSM];
@@ -342,7 +352,7 @@ window_attend_mfma_kernel(const bf16* __restrict__ q, long sq, const bf16* __res
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int j = k0 + 16 * kh + 4 * g + i;
-        const bool vis = j <= pq && j > pq - window;
+        const bool vis = j <= pq && j >= pq_lo;
         sc[kh][i] = vis ? st[kh][i] * scale : -INFINITY;
         tmax = fmaxf(tmax, sc[kh][i]);
       }
@@ -468,11 +478,13 @@ MX_API int mx_qk_norm_write(const void* q, long sq, const void* k, long sk, cons
 
 // q [T, H*D] (row stride sq), out [T, H*P] contiguous; cu [S+1] row bounds of the segments, pos [T]
 // positions, bt [S, btw] page tables; gate [T, >= H] slice (row stride sgate) or null.
+// chunked != 0: `window` is the block size of the chunked mask instead of a sliding window's length.
 // nsplit > 1 with a workspace ws (f32 [T, H, nsplit, P + 2]) and single-row segments: the key range of
 // each row is walked by nsplit blocks and merged (bf16 matrix-core form only; ignored otherwise).
 MX_API int mx_window_attend(const void* q, long sq, const void* cache, const int* cu, const int* pos, const int* bt,
-                            int btw, const void* gate, long sgate, int window, float scale, void* out, int dt, int S,
-                            int max_len, int H, int G, int D, int P, int nsplit, float* ws, hipStream_t st) {
+                            int btw, const void* gate, long sgate, int window, int chunked, float scale, void* out,
+                            int dt, int S, int max_len, int H, int G, int D, int P, int nsplit, float* ws,
+                            hipStream_t st) {
   if (S <= 0 || max_len <= 0) return 0;
   if (P > 64 * WA_CPL || G < 1 || H % G || window < 1) return (int)hipErrorInvalidValue;
   const int rep = H / G;
@@ -486,12 +498,12 @@ MX_API int mx_window_attend(const void* q, long sq, const void* cache, const int
     dim3 grid(nsplit > 1 ? nsplit : (max_len + QT - 1) / QT, G * ((rep + HB - 1) / HB), S);
     if (D <= 128 && P <= 128)
       window_attend_mfma_kernel<4, 8><<<grid, 256, lds, st>>>(
-          (const bf16*)q, sq, (const bf16*)cache, cu, pos, bt, btw, (const bf16*)gate, sgate, window, scale, (bf16*)out, H,
-          G, D, P, QT, HB, nsplit, ws);
+          (const bf16*)q, sq, (const bf16*)cache, cu, pos, bt, btw, (const bf16*)gate, sgate, window, chunked, scale,
+          (bf16*)out, H, G, D, P, QT, HB, nsplit, ws);
     else
       window_attend_mfma_kernel<8, 16><<<grid, 256, lds, st>>>(
-          (const bf16*)q, sq, (const bf16*)cache, cu, pos, bt, btw, (const bf16*)gate, sgate, window, scale, (bf16*)out, H,
-          G, D, P, QT, HB, nsplit, ws);
+          (const bf16*)q, sq, (const bf16*)cache, cu, pos, bt, btw, (const bf16*)gate, sgate, window, chunked, scale,
+          (bf16*)out, H, G, D, P, QT, HB, nsplit, ws);
     if (nsplit > 1) {
       dim3 g2(S, H);           // single-row segments: row index == segment index
       window_merge_kernel<<<g2, P >= 128 ? 128 : 64, 0, st>>>(ws, (const bf16*)gate, sgate, (bf16*)out, H, P, nsplit);
@@ -518,7 +530,7 @@ MX_API int mx_window_attend(const void* q, long sq, const void* cache, const int
   if (lds > 64 * 1024) return (int)hipErrorInvalidValue;
   dim3 grid((max_len + QT - 1) / QT, G * ((rep + HB - 1) / HB), S);
   MX_DISPATCH(dt, TT, window_attend_kernel<TT><<<grid, WA_WAVES * 64, lds, st>>>(
-      (const TT*)q, sq, (const TT*)cache, cu, pos, bt, btw, (const TT*)gate, sgate, window, scale, (TT*)out, H, G, D, P,
-      QT, HB, KT, ldk, ldv));
+      (const TT*)q, sq, (const TT*)cache, cu, pos, bt, btw, (const TT*)gate, sgate, window, chunked, scale, (TT*)out, H, G,
+      D, P, QT, HB, KT, ldk, ldv));
   MX_RETURN_LAUNCH();
 }

@@ -485,6 +485,7 @@ class ModelRunner:
         # (layered decoders come in arbitrary widths: they take the fused kernels only at the widths those
         # were measured at, multiples of 256, and logits + sampler otherwise)
         return (getattr(m, "tp_size", 1) == 1 and hasattr(m, "lm_weight") and h.dtype == torch.bfloat16
+                and getattr(m, "plain_logits", True)
                 and (not self.seg or h.shape[1] % 256 == 0) and ops.fused_lm_head_ok(h, m.lm_weight()))
 
     def _lm_tiled(self):

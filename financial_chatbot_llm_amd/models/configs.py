@@ -15,7 +15,7 @@ from typing import Dict, Optional
 @dataclass(frozen=True)
 class ModelConfig:
     name: str
-    arch: str                       # "llama" | "mixtral" | "bert" | "gezavik" | "sigudra"
+    arch: str                       # "llama" | "mixtral" | "bert" | "gezavik" | "sigudra" | "tukedra"
     vocab_size: int
     hidden_size: int
     num_layers: int
@@ -38,7 +38,10 @@ class ModelConfig:
     # as the checkpoint's config.json gives them; residual_mult scales each block's update
     layers: tuple = ()
     residual_mult: float = 1.0
-    embedding: Optional[Dict] = None    # layered decoders: extra embedding tables ({"bigram": {buckets, mul_prev, mul_cur}})
+    embedding: Optional[Dict] = None    # layered decoders: {"bigram": {buckets, mul_prev, mul_cur}} extra table, {"scale": s}
+    streams: int = 0                    # residual streams per token (hyper-connections); 0: one plain residual sum
+    logit_scale: float = 1.0            # logits <- head x * logit_scale ...
+    logit_softcap: float = 0.0          # ... then cap * tanh(logits / cap) (0: none)
 
     @property
     def q_size(self) -> int:
@@ -81,16 +84,20 @@ REGISTRY: Dict[str, ModelConfig] = {
 def _register_layered() -> None:
     from .gezavik import example_config
     from .sigudra import example_config as sigudra_config
+    from .tukedra import example_config as tukedra_config
     for name, kw in (("gezavik-tiny", dict(width=192, vocab=1024, heads=3, pattern="amAm")),
                      ("gezavik-1b", dict(width=2048, vocab=32768, heads=16, pattern="aMmAmMaM" * 2, scale_up=True))):
         REGISTRY[name] = layered_config(example_config(**kw), name)
     for name, kw in (("sigudra-tiny", dict(width=160, vocab=640, pattern="dGPd")),
                      ("sigudra-1b", dict(width=2048, vocab=32768, pattern="dGPgDpdG" * 2, scale_up=True))):
         REGISTRY[name] = layered_config(sigudra_config(**kw), name)
+    for name, kw in (("tukedra-tiny", dict(width=160, vocab=640, pattern="lRaL")),
+                     ("tukedra-1b", dict(width=2048, vocab=32768, pattern="lLRAlLRA" * 2, scale_up=True))):
+        REGISTRY[name] = layered_config(tukedra_config(**kw), name)
 
 
 def get_model_config(name: str) -> ModelConfig:
-    if name.startswith(("gezavik-", "sigudra-")) and name not in REGISTRY:
+    if name.startswith(("gezavik-", "sigudra-", "tukedra-")) and name not in REGISTRY:
         _register_layered()
     if name in REGISTRY:
         return REGISTRY[name]
@@ -125,12 +132,13 @@ def from_hf(path: str, name: Optional[str] = None) -> ModelConfig:
         top_k_experts=c.get("num_experts_per_tok", 0), bos_token_id=c.get("bos_token_id", 1), eos_token_ids=eos)
 
 
-LAYERED_ARCHS = ("gezavik", "sigudra")
+LAYERED_ARCHS = ("gezavik", "sigudra", "tukedra")
 
 
 def layered_config(c: Dict, name: Optional[str] = None) -> ModelConfig:
     """A layered decoder's ``config.json`` (``architecture``, ``layers``: type / mixer / mlp per layer,
-    ``norm.eps``, ``residual_mult``, ``embedding``, ``vocab``, ``width``) -> :class:`ModelConfig`.  The
+    ``norm.eps``, ``residual_mult``, ``embedding``, ``streams``, ``logit_scale``, ``logit_softcap``, ``vocab``,
+    ``width``) -> :class:`ModelConfig`.  The
     flat head fields hold the first attention layer's sizes (informational; the layers carry their own)."""
     arch = str(c["architecture"]).lower()
     if arch not in LAYERED_ARCHS:
@@ -138,9 +146,12 @@ def layered_config(c: Dict, name: Optional[str] = None) -> ModelConfig:
     layers = tuple(c["layers"])
     att = next((l["mixer"] for l in layers if "heads" in l["mixer"] and "kv_rank" in l["mixer"]), None)
     win = next((l["mixer"]["left"] for l in layers if "left" in l["mixer"]), None)
+    win = win or next((l["mixer"] for l in layers if l.get("type") == "attention"), None)
     heads = att["heads"] if att else (win["heads"] if win else 1)
     hd = (att["dim"] + att["rot_dim"]) if att else (win["dim"] if win else c["width"])
     ffs = [l["mlp"]["ff"] for l in layers if l.get("mlp") and l["mlp"].get("kind") == "dense"]
     return ModelConfig(name or arch, arch, c["vocab"], c["width"], len(layers), heads, 1, hd, max(ffs, default=0),
                        max_position=1 << 24, norm_eps=float(c["norm"]["eps"]), bos_token_id=0, eos_token_ids=(),
-                       layers=layers, residual_mult=float(c.get("residual_mult", 1.0)), embedding=c.get("embedding"))
+                       layers=layers, residual_mult=float(c.get("residual_mult", 1.0)), embedding=c.get("embedding"),
+                       streams=int(c.get("streams") or 0), logit_scale=float(c.get("logit_scale", 1.0)),
+                       logit_softcap=float(c.get("logit_softcap") or 0.0))

@@ -1,4 +1,4 @@
-"""Common part of the layered decoders (:mod:`.gezavik`, :mod:`.sigudra`): a ``config.json`` lists the
+"""Common part of the layered decoders (:mod:`.gezavik`, :mod:`.sigudra`, :mod:`.tukedra`): a ``config.json`` lists the
 layers, each with one sequence mixer of :mod:`.mixers` and optionally one feed-forward; the residual
 stream is f32 whatever the activation dtype; the checkpoint is the model directory itself (tensors
 ``embed``, ``l<i>.<norm>``, ``l<i>.mix.<name>``, ``l<i>.mlp.<name>``, ``final.norm``, ``head``; linear
@@ -38,6 +38,10 @@ class Layer:
 
     def norms(self):
         return self.norm_names
+
+    def extra_shapes(self) -> Dict[str, tuple]:
+        """Further per-layer tensors of the design: {name after the layer prefix: shape}."""
+        return {}
 
 
 class LayeredDecoder:
@@ -82,6 +86,7 @@ class LayeredDecoder:
         for l in self.layers:
             for n in l.norms():
                 s[f"{l.prefix}.{n}"] = (c.hidden_size,)
+            s.update({f"{l.prefix}.{k}": v for k, v in l.extra_shapes().items()})
             s.update({f"{l.prefix}.mix.{k}": v for k, v in l.mixer.shapes().items()})
             if l.ff is not None:
                 s.update({f"{l.prefix}.mlp.{k}": v for k, v in l.ff.shapes().items()})
@@ -93,6 +98,10 @@ class LayeredDecoder:
         randn = lambda: torch.randn(shape, generator=g, device=device)  # noqa: E731
         rand = lambda: torch.rand(shape, generator=g, device=device)  # noqa: E731
         leaf = name.rsplit(".", 1)[-1]
+        if ".hc" in name and leaf == "in":       # stream read weights: about an average of the streams
+            return (1.0 + 0.3 * randn()) / shape[0]
+        if ".hc" in name and leaf == "mix":      # stream mixing: near the identity
+            return torch.eye(shape[0], device=device) + 0.15 * randn()
         if leaf in ("norm1", "norm2", "norm", "out") and len(shape) == 1:
             return 1.0 + 0.1 * randn()
         if leaf == "A_log":

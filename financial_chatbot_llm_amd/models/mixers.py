@@ -17,7 +17,16 @@ normed input ``h`` and return a sublayer output, with their sizes and constants 
   convolved, block-diagonally gated diagonal recurrence).
 * :class:`ParallelMixer` -- two of the above side by side on the same input; the layer combines their
   RMS-normed outputs.
+* :class:`LightningMixer` -- linear attention with one fixed decay per head on SiLU-activated q, k, v,
+  an RMS norm over all heads and a sigmoid output gate.
+* :class:`RetentionMixer` -- the same recurrence on rotated q and k (half-split pairs), a weightless RMS
+  norm per head and a SiLU output gate.
+* :class:`ChunkAttentionMixer` -- softmax attention whose values are the keys as projected; biased q / k
+  projections, pairwise rotation with optionally scaled frequencies, weightless per-head RMS norm of q
+  and k after the rotation, and a chunked mask (a query sees the keys of its own block of positions).
 * :class:`DenseFF` -- up, activation, down; optionally gated (act(gate) * up).
+* :class:`TopSoftmaxRoutedFF` -- mixture of plain relu^2 experts, softmax over the chosen logits, plus a
+  shared expert.
 * :class:`RoutedFF` -- mixture of clamped gated experts with biased top-k choice, identity experts
   and an always-on shared expert.
 * :class:`InputScaledRoutedFF` -- mixture of gated experts chosen by independent sigmoid scores, the
@@ -333,6 +342,71 @@ class InputScaledRoutedFF:
         return mx.moe_combine(ys, pos.view(T, top).to(torch.int32), idx, ones, h, None, E)
 
 
+class TopSoftmaxRoutedFF:
+    """Mixture of ``experts`` plain feed-forwards W_down act(W_up h) (``act``: the square of relu, no
+    biases), ``top`` per token: router logits z = W_r h in f32, the ``top`` largest chosen (ties: the
+    lower index), weights = softmax over the chosen logits only; the output is the weighted sum of
+    the chosen experts' outputs plus, with a ``shared`` entry, an always-on expert of the same form."""
+
+    def __init__(self, spec: Dict, width: int, act: str = "relu2"):
+        r = spec["router"]
+        self.E, self.top = int(r["experts"]), int(r["top"])
+        self.F = int(spec["expert"]["ff"])
+        sh = spec.get("shared")
+        self.Fs = int(sh["ff"]) if sh else 0
+        self.act, self.width = act, width
+        self.in_rows = self.Fs                                            # the shared expert's up rows
+        if not 1 <= self.top <= self.E or act != "relu2":
+            raise ValueError("routed feed-forward: 1 <= top <= experts, activation relu2")
+
+    def shapes(self) -> Dict[str, tuple]:
+        s = {"router": (self.E, self.width)}
+        for e in range(self.E):
+            s.update({f"e{e}.up": (self.F, self.width), f"e{e}.down": (self.width, self.F)})
+        if self.Fs:
+            s.update({"shared.up": (self.Fs, self.width), "shared.down": (self.width, self.Fs)})
+        return s
+
+    def load(self, get: Getter, dtype) -> Optional[torch.Tensor]:
+        self.router = get("router").float().contiguous()
+        self.w1 = torch.stack([get(f"e{e}.up") for e in range(self.E)]).to(dtype).contiguous()        # [E, F, W]
+        self.w2 = torch.stack([get(f"e{e}.down") for e in range(self.E)]).to(dtype).contiguous()      # [E, W, F]
+        if not self.Fs:
+            return None
+        self.down_s = get("shared.down").to(dtype).contiguous()
+        return get("shared.up").to(dtype)
+
+    def num_bytes(self) -> int:
+        ts = [self.router, self.w1, self.w2] + ([self.down_s] if self.Fs else [])
+        return sum(t.numel() * t.element_size() for t in ts)
+
+    def forward(self, h: torch.Tensor, proj: Optional[torch.Tensor] = None, x32: Optional[torch.Tensor] = None) -> torch.Tensor:
+        T, W = h.shape
+        E, top, Fe = self.E, self.top, self.F
+        shared = F.linear(mx.relu2(proj[:, :self.Fs]), self.down_s) if self.Fs else None
+        wts, idx = mx.route_scores(F.linear(x32 if x32 is not None else h.float(), self.router), top, "softmax_top")
+        if T * top <= DENSE_MAX_PAIRS or _capturing(h):
+            up = torch.bmm(h.unsqueeze(0).expand(E, T, W), self.w1.transpose(1, 2)).view(E * T, Fe)
+            ys = torch.bmm(mx.relu2(up).view(E, T, Fe), self.w2.transpose(1, 2)).view(E * T, W)
+            rows = torch.arange(T, dtype=torch.int32, device=h.device)[:, None]
+            return mx.moe_combine(ys, (idx * T + rows).to(torch.int32), idx, wts, h, shared, E)
+        flat = idx.reshape(-1).long()
+        order = torch.argsort(flat, stable=True)
+        offs = [0] + torch.bincount(flat, minlength=E).cumsum(0).tolist()              # host read of the buckets
+        xs = h.index_select(0, order // top)
+        up = torch.empty((T * top, Fe), dtype=h.dtype, device=h.device)
+        live = [(e, offs[e], offs[e + 1]) for e in range(E) if offs[e + 1] > offs[e]]
+        for e, a, b in live:
+            torch.mm(xs[a:b], self.w1[e].t(), out=up[a:b])
+        act = mx.relu2(up)                                   # one activation launch over all buckets
+        ys = torch.empty((T * top, W), dtype=h.dtype, device=h.device)
+        for e, a, b in live:
+            torch.mm(act[a:b], self.w2[e].t(), out=ys[a:b])
+        pos = torch.empty_like(order)
+        pos[order] = torch.arange(order.numel(), device=order.device)
+        return mx.moe_combine(ys, pos.view(T, top).to(torch.int32), idx, wts, h, shared, E)
+
+
 def _f32(get: Getter, name: str) -> torch.Tensor:
     return get(name).float().contiguous()
 
@@ -535,6 +609,172 @@ class GatedLRUMixer:
         return F.linear(s, self.o)
 
 
+def _decays(spec: Dict, heads: int) -> torch.Tensor:
+    d = [float(v) for v in spec["decay"]]
+    if len(d) != heads or any(not 0.0 <= v <= 1.0 for v in d):
+        raise ValueError("decay: one value in [0, 1] per head")
+    return torch.tensor(d, dtype=torch.float32)
+
+
+class LightningMixer:
+    """Linear attention with one fixed decay per head: q = silu(W_q h), k = silu(W_k h) ([heads, dim]),
+    v = silu(W_v h) ([heads, vdim]); on the f32 state S [dim, vdim]: S <- decay_h S + k v^T, o = S^T q (no
+    other scale).  The concatenated heads are RMS-normed together with the weight ``norm``
+    [heads * vdim], multiplied by sigmoid(W_g h) and projected by W_o."""
+    kind = "lightning"
+    in_bias = None             # no bias on the stacked input projection
+
+    def __init__(self, spec: Dict, width: int, eps: float):
+        self.H, self.D, self.P = int(spec["heads"]), int(spec["dim"]), int(spec["vdim"])
+        self.decay = _decays(spec, self.H)
+        self.width, self.eps = width, eps
+        if self.D > 512:
+            raise ValueError("lightning: dim <= 512")
+        self.nq, self.nv = self.H * self.D, self.H * self.P
+        self.in_rows = 2 * self.nq + 2 * self.nv
+
+    def shapes(self) -> Dict[str, tuple]:
+        W = self.width
+        return {"q": (self.nq, W), "k": (self.nq, W), "v": (self.nv, W), "g": (self.nv, W), "o": (W, self.nv),
+                "norm": (self.nv,)}
+
+    def cache_spec(self):
+        return ("slots", {"S": (self.H, self.D, self.P)})
+
+    def load(self, get: Getter, dtype) -> torch.Tensor:
+        self.norm_w = _f32(get, "norm")
+        self.o = get("o").to(dtype).contiguous()
+        self.decay = self.decay.to(self.o.device)
+        return torch.cat([get("q"), get("k"), get("v"), get("g")], 0).to(dtype)
+
+    def num_bytes(self) -> int:
+        return self.o.numel() * self.o.element_size()
+
+    def forward(self, proj: torch.Tensor, positions: torch.Tensor, meta: AttentionMetadata, cache) -> torch.Tensor:
+        st = cache[1]
+        nq, nv = self.nq, self.nv
+        o = mx.decay_scan(proj[:, :nq], proj[:, nq:2 * nq], proj[:, 2 * nq:2 * nq + nv], self.decay, st["S"], meta.seg_cu,
+                          meta.seg_state, positions, self.H, self.D, self.P, act="silu", max_len=meta.seg_max_len)
+        gate = proj[:, 2 * nq + nv:2 * nq + 2 * nv]
+        return F.linear(mx.head_norm_gate(o, self.norm_w, self.eps, gate, 1, "sigmoid", proj.dtype), self.o)
+
+
+class _Rotary:
+    """The ``rot`` entry of a mixer spec: {dims, base, scaling?} -> frequencies (f32, on the device at load)
+    and the factor on cos and sin.  No entry: no rotation."""
+
+    def __init__(self, rot: Optional[Dict], dim: int):
+        self.dims = int(rot["dims"]) if rot else 0
+        if self.dims % 2 or self.dims > dim:
+            raise ValueError("rot.dims must be even and at most the head size")
+        self.freq, self.mscale = (mx.rope_freqs(self.dims, float(rot["base"]), rot.get("scaling"))
+                                  if self.dims else (None, 1.0))
+
+    def to(self, device):
+        if self.freq is not None:
+            self.freq = self.freq.to(device)
+
+
+class RetentionMixer:
+    """Linear attention with one fixed decay per head, no softmax and no denominator: q = W_q h,
+    k = W_k h ([heads, dim]), v = W_v h ([heads, vdim]); q and k rotated on their first rot.dims entries
+    (pair i is entries (i, i + dims/2), angle position * base^(-2i/dims)), then k times dim^-1/2;
+    S <- decay_h S + k v^T, o = S^T q on the f32 state.  Each head's o is divided by its root mean square
+    (no weight); the heads are multiplied by silu(W_g h) and projected by W_o."""
+    kind = "retention"
+    in_bias = None
+
+    def __init__(self, spec: Dict, width: int, eps: float):
+        self.H, self.D, self.P = int(spec["heads"]), int(spec["dim"]), int(spec["vdim"])
+        self.decay = _decays(spec, self.H)
+        self.rot = _Rotary(spec.get("rot"), self.D)
+        self.width, self.eps = width, eps
+        if self.D > 512:
+            raise ValueError("retention: dim <= 512")
+        self.nq, self.nv = self.H * self.D, self.H * self.P
+        self.in_rows = 2 * self.nq + 2 * self.nv
+
+    def shapes(self) -> Dict[str, tuple]:
+        W = self.width
+        return {"q": (self.nq, W), "k": (self.nq, W), "v": (self.nv, W), "g": (self.nv, W), "o": (W, self.nv)}
+
+    def cache_spec(self):
+        return ("slots", {"S": (self.H, self.D, self.P)})
+
+    def load(self, get: Getter, dtype) -> torch.Tensor:
+        self.o = get("o").to(dtype).contiguous()
+        self.decay = self.decay.to(self.o.device)
+        self.rot.to(self.o.device)
+        return torch.cat([get("q"), get("k"), get("v"), get("g")], 0).to(dtype)
+
+    def num_bytes(self) -> int:
+        return self.o.numel() * self.o.element_size()
+
+    def forward(self, proj: torch.Tensor, positions: torch.Tensor, meta: AttentionMetadata, cache) -> torch.Tensor:
+        st = cache[1]
+        nq, nv = self.nq, self.nv
+        # rotated q and k enter the recurrence: they stay f32
+        q, k = mx.rope_heads(proj[:, :nq], proj[:, nq:2 * nq], self.H, self.H, self.D, self.rot.freq, positions, "half",
+                             self.rot.mscale, k_scale=self.D ** -0.5, q_dtype=torch.float32, k_dtype=torch.float32)
+        o = mx.decay_scan(q, k, proj[:, 2 * nq:2 * nq + nv], self.decay, st["S"], meta.seg_cu, meta.seg_state, positions,
+                          self.H, self.D, self.P, max_len=meta.seg_max_len)
+        gate = proj[:, 2 * nq + nv:2 * nq + 2 * nv]
+        return F.linear(mx.head_norm_gate(o, None, self.eps, gate, self.H, "silu", proj.dtype), self.o)
+
+
+class ChunkAttentionMixer:
+    """Softmax attention with ``kv_heads`` key/value heads (query head h reads head h // (H/G)) whose
+    VALUES ARE THE KEYS as projected: q = W_q h + b_q, k = W_k h + b_k, v = k before norm and rotation.
+    q and k are rotated on their first rot.dims entries (pair i is entries (2i, 2i+1); frequencies
+    optionally scaled, see :func:`..ops.mixers.rope_freqs`), then each head is divided by its root mean
+    square over dim (no weight).  score = q . k * scale; the query at position i sees keys j <= i of
+    its own block, floor(j / mask.size) == floor(i / mask.size), blocks counted from position 0 (no
+    ``mask`` entry: plain causal); softmax; W_o on the concatenated heads.  The cache holds one row
+    [finished k | raw k] per token."""
+    kind = "attention"
+
+    def __init__(self, spec: Dict, width: int, eps: float):
+        self.H, self.G = int(spec["heads"]), int(spec.get("kv_heads", spec["heads"]))
+        self.D, self.P = int(spec["dim"]), int(spec.get("vdim", spec["dim"]))
+        if self.P != self.D:
+            raise ValueError("attention: the values are the keys, so vdim must equal dim")
+        self.rot = _Rotary(spec.get("rot"), self.D)
+        mask = spec.get("mask") or {}
+        self.chunk = int(mask["size"]) if mask.get("size") else 0
+        self.scale = float(spec["scale"]) if "scale" in spec else self.D ** -0.5
+        self.width, self.eps = width, eps
+        if self.H % self.G or self.D > 512:
+            raise ValueError("attention: heads must split into kv_heads; dim <= 512")
+        self.nq, self.nk = self.H * self.D, self.G * self.D
+        self.in_rows = self.nq + self.nk
+
+    def shapes(self) -> Dict[str, tuple]:
+        W = self.width
+        return {"q": (self.nq, W), "q.b": (self.nq,), "k": (self.nk, W), "k.b": (self.nk,), "o": (W, self.H * self.P)}
+
+    def cache_spec(self):
+        return ("rows", 2 * self.nk)
+
+    def load(self, get: Getter, dtype) -> torch.Tensor:
+        self.o = get("o").to(dtype).contiguous()
+        self.rot.to(self.o.device)
+        self.in_bias = torch.cat([get("q.b"), get("k.b")], 0).to(dtype).contiguous()
+        return torch.cat([get("q"), get("k")], 0).to(dtype)
+
+    def num_bytes(self) -> int:
+        return self.o.numel() * self.o.element_size()
+
+    def forward(self, proj: torch.Tensor, positions: torch.Tensor, meta: AttentionMetadata, cache) -> torch.Tensor:
+        rows = cache[1]
+        nq, nk = self.nq, self.nk
+        kraw = proj[:, nq:nq + nk]
+        q, _ = mx.rope_heads(proj[:, :nq], kraw, self.H, self.G, self.D, self.rot.freq, positions, "pairs",
+                             self.rot.mscale, norm_eps=self.eps, k_out=rows, slots=meta.slots, v=kraw)
+        o = mx.window_attend(q, rows, meta.seg_cu, positions, meta.seg_bt, self.chunk or (1 << 30), self.scale,
+                             meta.seg_max_len, self.H, self.G, self.D, self.P, chunked=bool(self.chunk))
+        return F.linear(o, self.o)
+
+
 class ParallelMixer:
     """Two mixers side by side reading the same input (``left``: windowed attention, ``right``: gated
     LRU block).  ``forward`` returns both outputs; the layer takes half the sum of their RMS norms
@@ -573,4 +813,5 @@ class ParallelMixer:
 
 MIXERS = {"mamba2": Mamba2Mixer, "latent_attention": LatentAttentionMixer, "channel_delta": ChannelDeltaMixer,
           "gla": GLAMixer, "window_attention": WindowAttentionMixer, "gated_lru": GatedLRUMixer,
-          "parallel": ParallelMixer}
+          "parallel": ParallelMixer, "lightning": LightningMixer, "retention": RetentionMixer,
+          "attention": ChunkAttentionMixer}

@@ -5,7 +5,11 @@ sliding window, clamped gated units, and biased top-k routing; and, for the sequ
 decoders, a hashed token-pair embedding, layer norm on the sublayer output fused with the residual
 add, matrix-state linear recurrences (gated linear attention, gated delta rule), a real-gated linear
 recurrent unit, sliding-window attention with grouped key/value heads over a paged [k | v] row cache,
-gated activations with a per-row scale and sigmoid top-k routing.
+gated activations with a per-row scale and sigmoid top-k routing; and, for decoders with several
+residual streams per token (hyper-connections), the fused stream update + read + RMS norm, a rotation
+of projected heads (two pair layouts, scaled frequencies, per-head RMS norm), matrix-state recurrences
+with one fixed decay per head, a chunked attention mask, top-k routing with a softmax over the chosen
+logits, and the logit scale / soft cap.
 
 Activations are bf16 or f32 (a model-wide choice); statistics, scores, softmax, recurrences and the
 residual stream are f32 either way.  CUDA(HIP) tensors run the kernels of ``libpenny_mixers.so``
@@ -458,18 +462,28 @@ def glu_act(gate: torch.Tensor, up: torch.Tensor, act: str, row_scale: Optional[
     return (_act(g, act) * u).to(gate.dtype)
 
 
+ROUTE_SCORES = {"softmax": 0, "sigmoid": 1, "softmax_top": 2}
+
+
 def route_scores(z: torch.Tensor, top: int, score: str = "sigmoid") -> Tuple[torch.Tensor, torch.Tensor]:
     """The ``top`` largest entries of each row of the f32 router logits ``z`` (ties: the lower index)
-    and their scores -- sigmoid(z), independent per expert, or softmax(z) -- not renormalised.
-    Returns (weights f32 [T, top], indices int32 [T, top])."""
+    and their scores: ``sigmoid`` (independent per expert) or ``softmax`` over all entries, neither
+    renormalised, or ``softmax_top``: the softmax over the chosen logits only.
+    Returns (weights f32 [T, top], indices int32 [T, top]), the largest first."""
     T, E = z.shape
     assert z.dtype == torch.float32
     if N.use_native(z):
         z = z.contiguous()
         w = torch.empty((T, top), dtype=torch.float32, device=z.device)
         i = torch.empty((T, top), dtype=torch.int32, device=z.device)
-        N.mcall("mx_route_scores", N.ptr(z), E, top, 1 if score == "sigmoid" else 0, N.ptr(w), N.ptr(i), T, N.stream())
+        N.mcall("mx_route_scores", N.ptr(z), E, top, ROUTE_SCORES[score], N.ptr(w), N.ptr(i), T, N.stream())
         return w, i
+    if score == "softmax_top":
+        # a stable sort: ties go to the lower index, as in the kernel
+        idx = torch.sort(z, dim=-1, descending=True, stable=True).indices[:, :top]
+        return torch.softmax(z.gather(1, idx), -1), idx.to(torch.int32)
+    if score not in ROUTE_SCORES:
+        raise ValueError(f"unknown routing score {score!r}")
     s = torch.sigmoid(z) if score == "sigmoid" else torch.softmax(z, -1)
     idx = torch.topk(s, top, dim=-1).indices
     return s.gather(1, idx), idx.to(torch.int32)
@@ -579,7 +593,8 @@ def matrix_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, a: torch.Tens
 def head_norm_gate(o: torch.Tensor, w: torch.Tensor, eps: float, gate: torch.Tensor, heads: int, act: str,
                    out_dtype: torch.dtype) -> torch.Tensor:
     """Every head's part of ``o`` [T, H*P] divided by its root mean square over P, times ``w`` [P]
-    (shared by the heads), times act(gate) [T, H*P]; ``act``: sigmoid | silu."""
+    (shared by the heads; None: no weight), times act(gate) [T, H*P]; ``act``: sigmoid | silu.  With
+    ``heads=1`` the whole row is normed at once with a weight per column."""
     T, n = o.shape
     P = n // heads
     if N.use_native(o):
@@ -588,7 +603,9 @@ def head_norm_gate(o: torch.Tensor, w: torch.Tensor, eps: float, gate: torch.Ten
                 gate.stride(0), _dt(gate), ACTS[act], N.ptr(out), _dt(out), T, heads, P, N.stream())
         return out
     v = o.float().view(T, heads, P)
-    v = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+    v = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)
+    if w is not None:
+        v = v * w.float()
     return (v.reshape(T, n) * _act(gate.float(), act)).to(out_dtype)
 
 
@@ -663,9 +680,11 @@ def qk_norm_write(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, qw: Optiona
 
 def window_attend(q: torch.Tensor, cache: torch.Tensor, cu: torch.Tensor, pos: torch.Tensor, bt: torch.Tensor,
                   window: int, scale: float, max_len: int, heads: int, kv_heads: int, dim: int, vdim: int,
-                  gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+                  gate: Optional[torch.Tensor] = None, chunked: bool = False) -> torch.Tensor:
     """Causal softmax attention of ``q`` [T, H*dim] over the cache rows [k: G*dim | v: G*vdim] of each
-    segment's pages: the query at position p sees keys j with 0 <= p - j < window; query head h
+    segment's pages: the query at position p sees keys j with 0 <= p - j < window, or -- ``chunked`` --
+    the keys j <= p with floor(j / window) == floor(p / window) (blocks of ``window`` positions counted
+    from the start of the sequence); query head h
     reads key/value head h // (H/G); score = q . k * scale, f32 softmax; head h's output is
     multiplied by sigmoid(gate[t, h]) when a gate [T, H] is given.  Returns [T, H*vdim]."""
     T = q.shape[0]
@@ -685,8 +704,8 @@ def window_attend(q: torch.Tensor, cache: torch.Tensor, cu: torch.Tensor, pos: t
                 ws = torch.empty((T, H, nsplit, P + 2), dtype=torch.float32, device=q.device)
         N.mcall("mx_window_attend", N.ptr(_rows(q)), q.stride(0), N.ptr(cache), N.ptr(cu), N.ptr(pos), N.ptr(bt), bt.shape[1],
                 N.ptr(_rows(gate)) if gate is not None else None, gate.stride(0) if gate is not None else 0,
-                int(min(window, 1 << 30)), float(scale), N.ptr(out), _dt(q), S, int(max_len), H, G, D, P, nsplit,
-                N.ptr(ws), N.stream())
+                int(min(window, 1 << 30)), 1 if chunked else 0, float(scale), N.ptr(out), _dt(q), S, int(max_len), H, G,
+                D, P, nsplit, N.ptr(ws), N.stream())
         return out
     out = torch.zeros((T, H, P), dtype=torch.float32)
     rows = cache.view(-1, Wr).float()
@@ -704,9 +723,205 @@ def window_attend(q: torch.Tensor, cache: torch.Tensor, cu: torch.Tensor, pos: t
         sc = torch.einsum("nhd,jhd->nhj", q[a:b].float().view(-1, H, D), keys) * scale
         p = pos[a:b].long()[:, None]
         j = torch.arange(ctx)[None]
-        vis = (j <= p) & (j > p - window)
+        vis = (j <= p) & ((j // window == p // window) if chunked else (j > p - window))
         sc = sc.masked_fill(~vis[:, None, :], float("-inf"))
         out[a:b] = torch.einsum("nhj,jhp->nhp", torch.softmax(sc, -1), vals)
     if gate is not None:
         out = out * torch.sigmoid(gate.float())[:, :, None]
     return out.reshape(T, H * P).to(q.dtype)
+
+
+# ----------------------------------------------------------------------------------------------
+# several residual streams per token (hyper-connections); logit scale and soft cap
+# ----------------------------------------------------------------------------------------------
+MAX_STREAMS = 8
+
+
+def embed_scaled(ids: torch.Tensor, table: torch.Tensor, scale: float = 1.0, copies: int = 1) -> torch.Tensor:
+    """``copies`` equal f32 streams [T, copies, W] of ``table[id] * scale``."""
+    T, (V, W) = ids.numel(), table.shape
+    if N.use_native(table):
+        out = torch.empty((T, copies, W), dtype=torch.float32, device=table.device)
+        N.mcall("mx_embed_scaled", N.ptr(ids.to(torch.int32).contiguous()), N.ptr(table), _dt(table), float(scale),
+                int(copies), N.ptr(out), T, W, V, N.stream())
+        return out
+    row = table[ids.long().clamp(0, V - 1)].float() * scale
+    return row[:, None, :].repeat(1, copies, 1).contiguous()
+
+
+def hyper_mix(x: torch.Tensor, y: Optional[torch.Tensor], mix: Optional[torch.Tensor], w_out: Optional[torch.Tensor],
+              w_in: torch.Tensor, w: Optional[torch.Tensor], eps: float,
+              out_dtype: torch.dtype = torch.bfloat16) -> Optional[torch.Tensor]:
+    """One pass over the streams ``x`` (f32 [T, S, W], in place) between two sublayers.  With the output
+    ``y`` [T, W] of the sublayer that just ran: x_t <- sum_s mix[s, t] x_s + w_out[t] * y for every
+    stream t at once (``mix`` f32 [S, S] indexed [from, to], ``w_out`` f32 [S]).  Then the next
+    sublayer's input u = sum_t w_in[t] x_t and its RMS norm u / sqrt(mean(u^2) + eps) * w in
+    ``out_dtype`` (``w`` None: the update only).  S = 1 with mix = w_out = w_in = 1 is the plain
+    pre-norm residual sum."""
+    T, S, W = x.shape
+    assert x.dtype == torch.float32 and x.is_contiguous()
+    if S > MAX_STREAMS:
+        raise ValueError(f"at most {MAX_STREAMS} residual streams are supported, got {S}")
+    if N.use_native(x):
+        out = torch.empty((T, W), dtype=out_dtype, device=x.device) if w is not None else None
+        N.mcall("mx_hyper_mix", N.ptr(x), N.ptr(_rows(y)) if y is not None else None, y.stride(0) if y is not None else 0,
+                _dt(y) if y is not None else 1, N.ptr(mix), N.ptr(w_out), N.ptr(w_in), N.ptr(w), float(eps), N.ptr(out),
+                _dt(out) if out is not None else 1, T, S, W, N.stream())
+        return out
+    if y is not None:
+        new = torch.einsum("st,nsw->ntw", mix.float(), x) + w_out.float()[None, :, None] * y.float()[:, None, :]
+        x.copy_(new)
+    if w is None:
+        return None
+    u = torch.einsum("t,ntw->nw", w_in.float(), x)
+    return (u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps) * w.float()).to(out_dtype)
+
+
+def logit_cap(logits: torch.Tensor, scale: float = 1.0, cap: float = 0.0) -> torch.Tensor:
+    """``logits`` <- cap * tanh(logits * scale / cap) in place (``cap`` <= 0: the scale only)."""
+    if scale == 1.0 and cap <= 0:
+        return logits
+    if N.use_native(logits):
+        assert logits.is_contiguous()
+        N.mcall("mx_logit_cap", N.ptr(logits), _dt(logits), float(scale), float(cap), logits.numel(), N.stream())
+        return logits
+    v = logits.float() * scale
+    if cap > 0:
+        v = cap * torch.tanh(v / cap)
+    return logits.copy_(v.to(logits.dtype))
+
+
+# ----------------------------------------------------------------------------------------------
+# rotation of projected heads
+# ----------------------------------------------------------------------------------------------
+def rope_freqs(dims: int, base: float, scaling: Optional[dict] = None, device=None) -> Tuple[torch.Tensor, float]:
+    """Frequencies f_i = base^(-2i / dims), i < dims / 2 (f32) and the factor on cos and sin.  With a
+    ``scaling`` entry {factor, original, fast, slow} (YaRN): with turn(t) = dims ln(original / (2 pi t)) /
+    (2 ln base), lo = max(floor(turn(fast)), 0), hi = min(ceil(turn(slow)), dims - 1) and
+    ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1) the frequency is f_i / factor * ramp_i +
+    f_i (1 - ramp_i) and cos and sin are multiplied by 0.1 ln(factor) + 1."""
+    import math
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    f = float(base) ** (-2.0 * i / dims)
+    m = 1.0
+    if scaling:
+        factor, orig = float(scaling["factor"]), float(scaling["original"])
+        turn = lambda t: dims * math.log(orig / (2 * math.pi * float(t))) / (2 * math.log(float(base)))  # noqa: E731
+        lo = max(math.floor(turn(scaling["fast"])), 0)
+        hi = min(math.ceil(turn(scaling["slow"])), dims - 1)
+        ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0, 1)
+        f = f / factor * ramp + f * (1 - ramp)
+        m = 0.1 * math.log(factor) + 1.0
+    return f.to(torch.float32).to(device).contiguous(), m
+
+
+def _rotate_heads(x: torch.Tensor, ang: torch.Tensor, rot: int, half: bool, m: float) -> torch.Tensor:
+    """x f32 [T, H, D]; ang f32 [T, rot / 2]."""
+    if rot == 0:
+        return x
+    c, s = (torch.cos(ang) * m)[:, None, :], (torch.sin(ang) * m)[:, None, :]
+    out = x.clone()
+    if half:
+        a, b = x[..., :rot // 2], x[..., rot // 2:rot]
+        out[..., :rot // 2] = a * c - b * s
+        out[..., rot // 2:rot] = b * c + a * s
+    else:
+        a, b = x[..., 0:rot:2], x[..., 1:rot:2]
+        out[..., 0:rot:2] = a * c - b * s
+        out[..., 1:rot:2] = b * c + a * s
+    return out
+
+
+def rope_heads(q: torch.Tensor, k: torch.Tensor, heads: int, kv_heads: int, dim: int, freq: Optional[torch.Tensor],
+               pos: torch.Tensor, layout: str = "pairs", mscale: float = 1.0, norm_eps: Optional[float] = None,
+               q_scale: float = 1.0, k_scale: float = 1.0, q_dtype: Optional[torch.dtype] = None,
+               k_out: Optional[torch.Tensor] = None, slots: Optional[torch.Tensor] = None,
+               v: Optional[torch.Tensor] = None, k_dtype: Optional[torch.dtype] = None):
+    """Per head of ``q`` [T, H*dim] and ``k`` [T, G*dim] (column slices): the first ``2 * len(freq)``
+    entries are rotated by the angle pos * freq_i (f32), pair i being entries (2i, 2i+1) for
+    ``layout="pairs"`` or (i, i + rot/2) for ``"half"``; (u, v) -> (u cos - v sin, v cos + u sin) with cos and
+    sin times ``mscale``; then, with ``norm_eps``, the head is divided by its root mean square over
+    ``dim`` (no weight); then times ``q_scale`` / ``k_scale``.  Returns (q', k'): q' [T, H*dim] in
+    ``q_dtype``; k' [T, G*dim] in ``k_dtype`` -- or, with ``k_out`` (paged cache rows [rows, G*dim + nv])
+    and ``slots`` [T], k' is written to row slots[t] (< 0: no write) followed by the raw values ``v``
+    [T, nv], and None is returned for it."""
+    T = q.shape[0]
+    H, G, D = heads, kv_heads, dim
+    rot = 2 * freq.numel() if freq is not None else 0
+    half = layout == "half"
+    if layout not in ("pairs", "half") or rot > D:
+        raise ValueError("rope_heads: layout is pairs | half and the rotated part must fit the head")
+    q_dtype = q_dtype or q.dtype
+    norm = norm_eps is not None
+    if N.use_native(q):
+        assert q.dtype == k.dtype and (v is None or v.dtype == q.dtype)
+        qo = torch.empty((T, H * D), dtype=q_dtype, device=q.device)
+        if k_out is None:
+            ko = torch.empty((T, G * D), dtype=k_dtype or k.dtype, device=q.device)
+            dst, sko, sl, nv = ko, G * D, None, 0
+        else:
+            nv = v.shape[1] if v is not None else 0
+            assert k_out.shape[-1] >= G * D + nv and k_out.stride(-1) == 1 and slots is not None
+            ko, dst, sko, sl = None, k_out, k_out.shape[-1], slots
+        N.mcall("mx_rope_heads", N.ptr(_rows(q)), q.stride(0), H, N.ptr(_rows(k)), k.stride(0), G, _dt(q), D, rot,
+                1 if half else 0, N.ptr(freq), float(mscale), N.ptr(pos), 1 if norm else 0, float(norm_eps or 0.0),
+                float(q_scale), float(k_scale), N.ptr(qo), _dt(qo), N.ptr(dst), sko, _dt(dst), N.ptr(sl),
+                N.ptr(_rows(v)) if v is not None else None, v.stride(0) if v is not None else 0, nv, T, N.stream())
+        return qo, ko
+    ang = pos.float()[:, None] * freq.float()[None, :] if rot else None
+
+    def prep(x, nh, sc):
+        x = _rotate_heads(x.float().reshape(T, nh, D), ang, rot, half, mscale)
+        if norm:
+            x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + norm_eps)
+        return (x * sc).reshape(T, nh * D)
+
+    qo = prep(q, H, q_scale).to(q_dtype)
+    kk = prep(k, G, k_scale)
+    if k_out is None:
+        return qo, kk.to(k_dtype or k.dtype)
+    rows = torch.cat([kk] + ([v.float()] if v is not None else []), 1).to(k_out.dtype)
+    ok = slots >= 0
+    k_out.view(-1, k_out.shape[-1])[slots[ok].long(), :rows.shape[1]] = rows[ok]
+    return qo, None
+
+
+# ----------------------------------------------------------------------------------------------
+# matrix-state recurrence with one fixed decay per head
+# ----------------------------------------------------------------------------------------------
+def decay_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, state: torch.Tensor,
+               cu: torch.Tensor, slot: torch.Tensor, pos: torch.Tensor, heads: int, dim: int, vdim: int,
+               act: str = "none", out_scale: float = 1.0, max_len: int = 0) -> torch.Tensor:
+    """Token-by-token f32 recurrence over a [dim, vdim] state per head with a constant decay per head:
+    S <- decay[h] S + act(k) act(v)^T, o = S^T act(q) * out_scale.  ``q``, ``k`` [T, H*dim] (one storage
+    type) and ``v`` [T, H*vdim] (possibly another) are column slices; ``act``: none | silu, applied to
+    all three; ``decay`` f32 [H]; ``state`` f32 [slots, H, dim, vdim], read unless the segment starts at
+    position 0, then replaced.  Returns o f32 [T, H*vdim]."""
+    T = q.shape[0]
+    H, D, P = heads, dim, vdim
+    S = cu.numel() - 1
+    assert q.dtype == k.dtype and q.shape[1] == H * D and k.shape[1] == H * D and v.shape[1] == H * P
+    assert decay.dtype == torch.float32 and decay.numel() == H and act in ("none", "silu")
+    if N.use_native(q):
+        out = torch.empty((T, H * P), dtype=torch.float32, device=q.device)
+        N.mcall("mx_decay_scan", N.ptr(_rows(q)), q.stride(0), N.ptr(_rows(k)), k.stride(0), _dt(q), N.ptr(_rows(v)),
+                v.stride(0), _dt(v), ACTS[act], N.ptr(decay), float(out_scale), N.ptr(state), N.ptr(cu), N.ptr(slot),
+                N.ptr(pos), N.ptr(out), S, T, int(max_len), H, D, P, N.stream())
+        return out
+    out = torch.zeros((T, H * P), dtype=torch.float32)
+    cul, sll, pl = cu.tolist(), slot.tolist(), pos.tolist()
+    g = decay.float()[:, None, None]
+    for s in range(S):
+        r0, r1 = cul[s], cul[s + 1]
+        if sll[s] < 0 or r1 <= r0:
+            continue
+        n = r1 - r0
+        qq = _act(q[r0:r1].float(), act).view(n, H, D)
+        kk = _act(k[r0:r1].float(), act).view(n, H, D)
+        vv = _act(v[r0:r1].float(), act).view(n, H, P)
+        St = torch.zeros((H, D, P)) if pl[r0] == 0 else state[sll[s]].clone()
+        for t in range(n):
+            St = g * St + kk[t][:, :, None] * vv[t][:, None, :]
+            out[r0 + t] = (torch.einsum("hdp,hd->hp", St, qq[t]) * out_scale).reshape(-1)
+        state[sll[s]] = St
+    return out
