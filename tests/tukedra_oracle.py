@@ -109,16 +109,15 @@ def attention(h, sd, p, m, eps, pos):
     q = rms(rotate(q, pos, m.get("rot"), "pairs"), eps)
     k = rms(rotate(k, pos, m.get("rot"), "pairs"), eps)
     rep = H // G
-    out = torch.zeros((n, H, D), dtype=F64)
+    kk, vv = k.repeat_interleave(rep, 1), v.repeat_interleave(rep, 1)        # query head h reads head h // rep
+    sc = torch.einsum("ihd,jhd->hij", q, kk) * float(m["scale"])
     size = (m.get("mask") or {}).get("size")
-    for i in range(n):
-        pi = int(pos[i])
-        js = [j for j in range(i + 1) if size is None or int(pos[j]) // size == pi // size]
-        for hh in range(H):
-            g = hh // rep
-            sc = torch.stack([(q[i, hh] * k[j, g]).sum() for j in js]) * float(m["scale"])
-            w = torch.softmax(sc, 0)
-            out[i, hh] = sum(w[a] * v[j, g] for a, j in enumerate(js))
+    pi, pj = pos[:, None], pos[None, :]
+    seen = pj <= pi
+    if size is not None:
+        seen = seen & (pj // size == pi // size)
+    w = torch.softmax(sc.masked_fill(~seen[None], float("-inf")), -1)
+    out = torch.einsum("hij,jhd->ihd", w, vv)
     return out.reshape(n, H * D) @ _w(sd, p + "o").T
 
 
@@ -188,3 +187,13 @@ def forward(cfg: Dict, sd: Dict[str, torch.Tensor], tokens, capture: Optional[li
     if cap:
         logits = float(cap) * torch.tanh(logits / float(cap))
     return logits
+
+
+def greedy(cfg: Dict, sd: Dict[str, torch.Tensor], prompt: List[int], n: int) -> List[int]:
+    """``n`` greedy tokens after ``prompt``, each from a whole-sequence forward pass."""
+    toks, out = list(prompt), []
+    for _ in range(n):
+        nxt = int(forward(cfg, sd, toks)[-1].argmax())
+        out.append(nxt)
+        toks.append(nxt)
+    return out
