@@ -1,6 +1,6 @@
 """Times the sequence-mixer kernels (``ops.mixers``) at the layer shapes of a hybrid decoder.
 
-    python -m financial_chatbot_llm_amd.bench.mixer_kernels [--width 2048] [--design gezavik|sigudra]
+    python -m financial_chatbot_llm_amd.bench.mixer_kernels [--width 2048] [--design gezavik|sigudra|tukedra]
 
 Two step shapes: a prefill step of two 2048-token prompts and a decode step of 64 single rows at
 depth 1024.  Shapes follow ``models.gezavik.example_config(scale_up=True)``: Mamba-2 with inner =
@@ -9,7 +9,10 @@ kv_rank 256, rot_dim 32, window 1024.  One JSON line per kernel and shape (micro
 arithmetic or byte rate the time corresponds to).  ``--design sigudra``: the kernels of that design at
 ``models.sigudra.example_config(scale_up=True)`` shapes (width / 128 heads of key and value size 128
 for the delta rule and the windowed attention with 4 query heads per key/value head, 64-wide keys for
-gated linear attention, a gated LRU as wide as the model, window 1024).
+gated linear attention, a gated LRU as wide as the model, window 1024).  ``--design tukedra``: that
+design's kernels at ``models.tukedra.example_config(scale_up=True)`` shapes (width / 128 heads; lightning
+128 x 128 with the SiLU at staging, retention 64 x 128 on rotated f32 q and k, chunk-masked attention with
+128-wide heads, 4 query heads per key/value head and blocks of 1024 positions; two residual streams).
 """
 from __future__ import annotations
 
@@ -114,13 +117,79 @@ def sigudra(width: int) -> int:
     return 0
 
 
+def tukedra(width: int) -> int:
+    dev = "cuda"
+    H, D, P, size, S2 = max(width // 128, 2), 128, 128, 1024, 2
+    G = max(H // 4, 1)
+    out = lambda **kw: print(json.dumps(kw), flush=True)  # noqa: E731
+    for name, lens, start, cu, pos, slot in _steps(dev):
+        S, T, ml = len(lens), sum(lens), max(lens)
+        # lightning: one launch, SiLU while the rows are staged
+        qkv = torch.randn(T, 2 * H * D + H * P, device=dev).bfloat16() * 0.3
+        decay = torch.linspace(0.9, 0.999, H, device=dev)
+        st = torch.zeros(S, H, D, P, device=dev)
+        us = _time(lambda: mx.decay_scan(qkv[:, :H * D], qkv[:, H * D:2 * H * D], qkv[:, 2 * H * D:], decay, st, cu, slot, pos,
+                                         H, D, P, act="silu", max_len=ml), 5)
+        out(shape=name, kernel="decay_scan lightning", us=round(us, 1), f32_TFLOP_per_s=round(T * H * D * P * 5 / us / 1e6, 2),
+            state_TB_per_s=round(S * H * D * P * 8 / us / 1e6, 2))
+        # retention: rotation of q and k into f32, then the scan
+        Dr = 64
+        freq, ms = mx.rope_freqs(Dr, 10000.0, device=dev)
+        q2 = torch.randn(T, 2 * H * Dr + H * P, device=dev).bfloat16() * 0.3
+        us = _time(lambda: mx.rope_heads(q2[:, :H * Dr], q2[:, H * Dr:2 * H * Dr], H, H, Dr, freq, pos, "half", ms,
+                                         k_scale=Dr ** -0.5, q_dtype=torch.float32, k_dtype=torch.float32))
+        out(shape=name, kernel="rope_heads retention", us=round(us, 1), TB_per_s=round(T * 2 * H * Dr * 6 / us / 1e6, 2))
+        qf, kf = mx.rope_heads(q2[:, :H * Dr], q2[:, H * Dr:2 * H * Dr], H, H, Dr, freq, pos, "half", ms, k_scale=Dr ** -0.5,
+                               q_dtype=torch.float32, k_dtype=torch.float32)
+        st2 = torch.zeros(S, H, Dr, P, device=dev)
+        us = _time(lambda: mx.decay_scan(qf, kf, q2[:, 2 * H * Dr:], decay, st2, cu, slot, pos, H, Dr, P, max_len=ml), 5)
+        out(shape=name, kernel="decay_scan retention", us=round(us, 1), f32_TFLOP_per_s=round(T * H * Dr * P * 5 / us / 1e6, 2),
+            state_TB_per_s=round(S * H * Dr * P * 8 / us / 1e6, 2))
+        o = torch.randn(T, H * P, device=dev)
+        gt = torch.randn(T, H * P, device=dev).bfloat16()
+        nw = torch.ones(H * P, device=dev)
+        us = _time(lambda: mx.head_norm_gate(o, nw, 1e-5, gt, 1, "sigmoid", torch.bfloat16))
+        out(shape=name, kernel="head_norm_gate all heads", us=round(us, 1), TB_per_s=round(T * H * P * 8 / us / 1e6, 2))
+        us = _time(lambda: mx.head_norm_gate(o, None, 1e-5, gt, H, "silu", torch.bfloat16))
+        out(shape=name, kernel="head_norm_gate per head", us=round(us, 1), TB_per_s=round(T * H * P * 8 / us / 1e6, 2))
+        # attention: rotation + per-head norm + cache write, then the chunk-masked attention
+        pages = (start + ml + 63) // 64
+        cache = torch.randn(S * pages * 64, 2 * G * D, device=dev).bfloat16()
+        bt = torch.arange(S * pages, dtype=torch.int32, device=dev).view(S, pages).contiguous()
+        qk = torch.randn(T, (H + G) * D, device=dev).bfloat16()
+        fa, ma = mx.rope_freqs(64, 10000.0, {"factor": 4.0, "fast": 32.0, "original": 4096, "slow": 1.0}, device=dev)
+        slots = (bt[:, None, :].expand(S, ml, pages).reshape(-1, pages).gather(1, (pos // 64).long()[:, None])[:, 0] * 64
+                 + pos % 64).to(torch.int32)
+        us = _time(lambda: mx.rope_heads(qk[:, :H * D], qk[:, H * D:], H, G, D, fa, pos, "pairs", ma, norm_eps=1e-5,
+                                         k_out=cache, slots=slots, v=qk[:, H * D:]))
+        out(shape=name, kernel="rope_heads attention", us=round(us, 1),
+            TB_per_s=round(T * (2 * H * D + 3 * G * D) * 2 / us / 1e6, 2))
+        qn, _ = mx.rope_heads(qk[:, :H * D], qk[:, H * D:], H, G, D, fa, pos, "pairs", ma, norm_eps=1e-5, k_out=cache,
+                              slots=slots, v=qk[:, H * D:])
+        us = _time(lambda: mx.window_attend(qn, cache, cu, pos, bt, size, 1.0, ml, H, G, D, P, chunked=True), 5)
+        pairs = sum(p % size + 1 for n in lens for p in range(start, start + n))
+        keys = sum(max(p % size + 1 for p in range(start, start + n)) for n in lens)
+        out(shape=name, kernel="window_attend chunked", us=round(us, 1),
+            bf16_TFLOP_per_s=round(pairs * H * 2 * (D + P) / us / 1e6, 1),
+            cache_TB_per_s=round(keys * G * (D + P) * 2 / us / 1e6, 3))
+        x = torch.randn(T, S2, width, device=dev)
+        y = torch.randn(T, width, device=dev).bfloat16()
+        mix, wo, wi = torch.eye(S2, device=dev), torch.ones(S2, device=dev), torch.ones(S2, device=dev) / S2
+        w = torch.ones(width, device=dev)
+        us = _time(lambda: mx.hyper_mix(x, y, mix, wo, wi, w, 1e-5, torch.bfloat16))
+        out(shape=name, kernel="hyper_mix 2 streams", us=round(us, 1), TB_per_s=round(T * width * (8 * S2 + 4) / us / 1e6, 2))
+    return 0
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--width", type=int, default=2048)
-    ap.add_argument("--design", default="gezavik", choices=["gezavik", "sigudra"])
+    ap.add_argument("--design", default="gezavik", choices=["gezavik", "sigudra", "tukedra"])
     a = ap.parse_args(argv)
     if a.design == "sigudra":
         return sigudra(a.width)
+    if a.design == "tukedra":
+        return tukedra(a.width)
     dev = "cuda"
     H, P, Ns, G, K = 2 * a.width // 64, 64, 128, 2, 4
     C = H * P + 2 * G * Ns

@@ -2,6 +2,7 @@
 
     python bench.py --model-throughput gezavik [--mt-widths 1024,2048,4096]
     python bench.py --model-throughput sigudra          # beside Gezavik, its closest relative here
+    python bench.py --model-throughput tukedra          # beside Sigudra, its closest relative here
     python -m financial_chatbot_llm_amd.bench.model_throughput --mt-only gezavik-w2048
 
 For each width a Gezavik model (random weights, 8 layers: latent attention and Mamba-2 mixers, dense
@@ -84,6 +85,17 @@ def register_sigudra(width: int, vocab: int = 32768) -> List[str]:
     return [name, register(width, vocab)[0]]
 
 
+def register_tukedra(width: int, vocab: int = 32768) -> List[str]:
+    """Register ``tukedra-w<width>`` (8 layers ``lLRalLrA``: lightning and retention scans, chunk-masked
+    attention; dense and routed feed-forwards; two residual streams) and the Sigudra model of the same
+    width, depth and vocabulary (within 2 % of the same parameter count); returns the two names."""
+    from ..models.configs import REGISTRY, layered_config
+    from ..models.tukedra import example_config
+    name = f"tukedra-w{width}"
+    REGISTRY[name] = layered_config(example_config(width=width, vocab=vocab, pattern="lLRalLrA", scale_up=True), name)
+    return [name, register_sigudra(width, vocab)[0]]
+
+
 def _tokens(n: int, vocab: int, seed: int) -> List[int]:
     g = torch.Generator().manual_seed(seed)
     return torch.randint(5, vocab - 300, (n,), generator=g).tolist()
@@ -155,7 +167,7 @@ def run(a) -> int:
     names: List[str] = []
     design = getattr(a, "model_throughput", "") or "gezavik"
     for w in (int(x) for x in a.mt_widths.split(",") if x):
-        names += register_sigudra(w) if design == "sigudra" else register(w)
+        names += {"sigudra": register_sigudra, "tukedra": register_tukedra}.get(design, register)(w)
     if a.mt_only:
         names = [n for n in names if n == a.mt_only]
     for n in names:
@@ -166,7 +178,7 @@ def run(a) -> int:
 
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser()
-    ap.add_argument("--model-throughput", default="gezavik", choices=["gezavik", "sigudra"])
+    ap.add_argument("--model-throughput", default="gezavik", choices=["gezavik", "sigudra", "tukedra"])
     add_arguments(ap)
     return run(ap.parse_args(argv))
 

@@ -51,7 +51,7 @@ def example_config(width: int = 160, vocab: int = 640, pattern: str = "lRaL", sc
                "rot": {"base": 10000.0, "dims": 64, "scaling": {"factor": 4.0, "fast": 32.0, "original": 4096, "slow": 1.0}},
                "scale": 1.0, "vdim": 128}
         dense = {"ff": 3 * width, "kind": "dense"}
-        moe = {"expert": {"ff": width // 2}, "kind": "moe", "router": {"experts": 32, "top": 4}, "shared": {"ff": width}}
+        moe = {"expert": {"ff": 3 * width // 4}, "kind": "moe", "router": {"experts": 32, "top": 4}, "shared": {"ff": width}}
     else:
         lig = {"decay": [0.7, 0.95, 0.995], "dim": 24, "heads": 3, "vdim": 20}
         ret = {"decay": [0.9, 0.99], "dim": 20, "heads": 2, "rot": {"base": 5000.0, "dims": 12}, "vdim": 28}
