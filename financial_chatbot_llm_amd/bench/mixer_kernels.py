@@ -12,7 +12,7 @@ for the delta rule and the windowed attention with 4 query heads per key/value h
 gated linear attention, a gated LRU as wide as the model, window 1024).  ``--design tukedra``: that
 design's kernels at ``models.tukedra.example_config(scale_up=True)`` shapes (width / 128 heads; lightning
 128 x 128 with the SiLU at staging, retention 64 x 128 on rotated f32 q and k, chunk-masked attention with
-128-wide heads, 4 query heads per key/value head and blocks of 1024 positions; two residual streams).
+128-wide heads, 4 query heads per key/value head and blocks of 2048 positions; two residual streams).
 """
 from __future__ import annotations
 
@@ -119,7 +119,7 @@ def sigudra(width: int) -> int:
 
 def tukedra(width: int) -> int:
     dev = "cuda"
-    H, D, P, size, S2 = max(width // 128, 2), 128, 128, 1024, 2
+    H, D, P, size, S2 = max(width // 128, 2), 128, 128, 2048, 2
     G = max(H // 4, 1)
     out = lambda **kw: print(json.dumps(kw), flush=True)  # noqa: E731
     for name, lens, start, cu, pos, slot in _steps(dev):

@@ -129,13 +129,9 @@ matrix_scan_kernel(const TQ* __restrict__ q, long sq, const TQ* __restrict__ k, 
       const int t = e / DP, d = e - t * DP;
       const long row = r0 + min(t0 + t, n - 1);
       const int dc = min(d, D - 1);
-      if (FIXED) {
+      if (FIXED) {         // raw values: the activation waits until they are stored to LDS, so the loads stay in flight
         pq[i] = ldf(q + row * sq + kvh * D + dc);
         pk[i] = ldf(k + row * sk + kvh * D + dc);
-        if (fact == 1) {
-          pq[i] = mx_silu(pq[i]);
-          pk[i] = mx_silu(pk[i]);
-        }
       } else if (ONE) {       // no prep pass ran: the decay from its pre-activation here, the unit norms after staging
         pq[i] = ldf(q + row * sq + kvh * D + dc);
         pk[i] = ldf(k + row * sk + kvh * D + dc);
@@ -155,7 +151,6 @@ matrix_scan_kernel(const TQ* __restrict__ q, long sq, const TQ* __restrict__ k, 
       const long vi = (long)(r0 + min(t0 + t, n - 1)) * sv + h * P + min(c0 + c, P - 1);
       if (FIXED) {
         pv[i] = ld_code(v, vcode, vi);
-        if (fact == 1) pv[i] = mx_silu(pv[i]);
       } else {
         pv[i] = ldf(v + vi);
       }
@@ -173,15 +168,20 @@ matrix_scan_kernel(const TQ* __restrict__ q, long sq, const TQ* __restrict__ k, 
       const int e = tid + 256 * i;
       if (e < TB * DP) {
         const bool live = (e % DP) < D;
-        qs[e] = live ? pq[i] : 0.f;
-        ks[e] = live ? pk[i] : 0.f;
+        if (FIXED && fact == 1) {
+          qs[e] = live ? mx_silu(pq[i]) : 0.f;
+          ks[e] = live ? mx_silu(pk[i]) : 0.f;
+        } else {
+          qs[e] = live ? pq[i] : 0.f;
+          ks[e] = live ? pk[i] : 0.f;
+        }
         if (!FIXED) gs[e] = live ? pg[i] : 1.f;
       }
     }
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int e = tid + 256 * i;
-      if (e < TB * CB) vs[e] = (c0 + e % CB) < P ? pv[i] : 0.f;
+      if (e < TB * CB) vs[e] = (c0 + e % CB) < P ? ((FIXED && fact == 1) ? mx_silu(pv[i]) : pv[i]) : 0.f;
     }
     if (DELTA && tid < TB) bs[tid] = pb;
     __syncthreads();

@@ -15,7 +15,7 @@
 
 namespace {
 
-constexpr int HC_MAX = 8;          // streams
+constexpr int HC_LIMIT = 16;       // streams
 
 template <typename T>
 __global__ void embed_scaled_kernel(const int* __restrict__ ids, const T* __restrict__ table, float scale, int copies,
@@ -30,8 +30,8 @@ __global__ void embed_scaled_kernel(const int* __restrict__ ids, const T* __rest
   }
 }
 
-// one block per token; the row u lives in LDS (W floats)
-template <typename TA, typename TO>
+// one block per token; the row u lives in LDS (W floats); HC_MAX: streams padded to a compile-time count
+template <typename TA, typename TO, int HC_MAX>
 __global__ void hyper_mix_kernel(float* __restrict__ x, const TA* __restrict__ y, long sy, const float* __restrict__ mix,
                                  const float* __restrict__ wout, const float* __restrict__ win,
                                  const float* __restrict__ w, float eps, TO* __restrict__ out, int S, int W) {
@@ -103,30 +103,25 @@ rope_heads_kernel(const TI* __restrict__ q, long sq, int Hq, const TI* __restric
     const TI* src = isq ? q + t * sq + (long)head * D : k + t * sk + (long)(head - Hq) * D;
     if (!isq && krow < 0) continue;          // wave-uniform
     float ss = 0.f;
-    for (int d = lane; d < D; d += 64) {
-      float val = ldf(src + d);
-      if (d < rot) {
-        int i, partner;
-        bool first;
-        if (half) {
-          first = d < hr;
-          i = first ? d : d - hr;
-          partner = first ? d + hr : d - hr;
-        } else {
-          first = (d & 1) == 0;
-          i = d >> 1;
-          partner = d ^ 1;
-        }
-        float sn, cs;
-        sincosf(p * freq[i], &sn, &cs);
-        sn *= mscale;
-        cs *= mscale;
-        const float other = ldf(src + partner);
-        val = first ? val * cs - other * sn : val * cs + other * sn;
-      }
+    for (int i = lane; i < hr; i += 64) {    // a lane owns whole pairs: one sine and cosine per pair
+      const int a = half ? i : 2 * i, b = half ? i + hr : 2 * i + 1;
+      float sn, cs;
+      sincosf(p * freq[i], &sn, &cs);
+      sn *= mscale;
+      cs *= mscale;
+      const float u = ldf(src + a), w = ldf(src + b);
+      const float ra = u * cs - w * sn, rb = w * cs + u * sn;
+      mine[a] = ra;
+      mine[b] = rb;
+      ss += ra * ra + rb * rb;
+    }
+    for (int d = rot + lane; d < D; d += 64) {
+      const float val = ldf(src + d);
       mine[d] = val;
       ss += val * val;
     }
+    // the copy-out below reads entries other lanes wrote
+    __builtin_amdgcn_wave_barrier();
     float f = isq ? qscale : kscale;
     if (norm) f *= 1.0f / sqrtf(mx_wave_sum(ss) / (float)D + eps);
     if (isq) {
@@ -170,12 +165,19 @@ MX_API int mx_hyper_mix(float* x, const void* y, long sy, int dt_y, const float*
                         const float* win, const float* w, float eps, void* out, int dt_out, int T, int S, int W,
                         hipStream_t st) {
   if (T <= 0) return 0;
-  if (S < 1 || S > HC_MAX || (size_t)W * sizeof(float) > 60 * 1024 || win == nullptr ||
+  if (S < 1 || S > HC_LIMIT || (size_t)W * sizeof(float) > 60 * 1024 || win == nullptr ||
       (y != nullptr && (mix == nullptr || wout == nullptr)))
     return (int)hipErrorInvalidValue;
   const int nt = W >= 1024 ? 512 : 256;
-  MX_DISPATCH(dt_y, TA, MX_DISPATCH(dt_out, TO, hyper_mix_kernel<TA, TO><<<T, nt, (size_t)W * sizeof(float), st>>>(
-      x, (const TA*)y, sy, mix, wout, win, w, eps, (TO*)out, S, W)));
+  const size_t lds = (size_t)W * sizeof(float);
+#define HYPER_LAUNCH(HC)                                                                                        \
+  MX_DISPATCH(dt_y, TA, MX_DISPATCH(dt_out, TO, hyper_mix_kernel<TA, TO, HC><<<T, nt, lds, st>>>(                \
+      x, (const TA*)y, sy, mix, wout, win, w, eps, (TO*)out, S, W)))
+  if (S <= 2) HYPER_LAUNCH(2);
+  else if (S <= 4) HYPER_LAUNCH(4);
+  else if (S <= 8) HYPER_LAUNCH(8);
+  else HYPER_LAUNCH(16);
+#undef HYPER_LAUNCH
   MX_RETURN_LAUNCH();
 }
 

@@ -47,7 +47,7 @@ def example_config(width: int = 160, vocab: int = 640, pattern: str = "lRaL", sc
         lig = {"decay": [1.0 - 2.0 ** (-3 - 5 * h / max(H - 1, 1)) for h in range(H)], "dim": 128, "heads": H, "vdim": 128}
         ret = {"decay": [1.0 - 2.0 ** (-5 - 4 * h / max(H - 1, 1)) for h in range(H)], "dim": 64, "heads": H,
                "rot": {"base": 10000.0, "dims": 64}, "vdim": 128}
-        att = {"dim": 128, "heads": H, "kv_heads": max(H // 4, 1), "mask": {"size": 1024},
+        att = {"dim": 128, "heads": H, "kv_heads": max(H // 4, 1), "mask": {"size": 2048},
                "rot": {"base": 10000.0, "dims": 64, "scaling": {"factor": 4.0, "fast": 32.0, "original": 4096, "slow": 1.0}},
                "scale": 1.0, "vdim": 128}
         dense = {"ff": 3 * width, "kind": "dense"}

@@ -734,7 +734,7 @@ def window_attend(q: torch.Tensor, cache: torch.Tensor, cu: torch.Tensor, pos: t
 # ----------------------------------------------------------------------------------------------
 # several residual streams per token (hyper-connections); logit scale and soft cap
 # ----------------------------------------------------------------------------------------------
-MAX_STREAMS = 8
+MAX_STREAMS = 16
 
 
 def embed_scaled(ids: torch.Tensor, table: torch.Tensor, scale: float = 1.0, copies: int = 1) -> torch.Tensor:

@@ -138,7 +138,7 @@ def test_stream_sum_after_every_layer(device):
 
 
 @pytest.mark.parametrize("device", DEVICES)
-@pytest.mark.parametrize("streams", [0, 1, 2, 5, 8])
+@pytest.mark.parametrize("streams", [0, 1, 2, 5, 16])
 def test_stream_counts(device, streams):
     """No ``streams`` entry is the plain residual sum (no hc tensors at all); one stream still has its
     read, write and mix weights."""
@@ -515,7 +515,7 @@ def test_rotation_layouts_norm_and_cache_rows(device, layout):
 
 
 @pytest.mark.parametrize("device", DEVICES)
-@pytest.mark.parametrize("S", [1, 3, 8])
+@pytest.mark.parametrize("S", [1, 2, 3, 8, 13])
 def test_stream_update_read_and_norm(device, S):
     """x_t <- sum_s mix[s, t] x_s + out[t] y with mix indexed [from, to] (an asymmetric mix shows a
     transposed read), all streams from the OLD ones, then the read with the next weights and its norm."""
@@ -631,7 +631,7 @@ def test_registry_and_config_errors():
     with pytest.raises(ValueError):
         TukedraModel(layered_config(bad, "bad"), device="cpu")
     bad = copy.deepcopy(example_config())
-    bad["streams"] = 9
+    bad["streams"] = 17
     with pytest.raises(ValueError):
         TukedraModel(layered_config(bad, "bad"), device="cpu")
     m = TukedraModel(layered_config(example_config(), "ok"), device="cpu")
