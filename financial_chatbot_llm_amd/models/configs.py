@@ -91,7 +91,7 @@ def _register_layered() -> None:
     for name, kw in (("sigudra-tiny", dict(width=160, vocab=640, pattern="dGPd")),
                      ("sigudra-1b", dict(width=2048, vocab=32768, pattern="dGPgDpdG" * 2, scale_up=True))):
         REGISTRY[name] = layered_config(sigudra_config(**kw), name)
-    for name, kw in (("tukedra-tiny", dict(width=160, vocab=640, pattern="lRaL")),
+    for name, kw in (("tukedra-tiny", dict(width=160, vocab=768, pattern="lRaL")),
                      ("tukedra-1b", dict(width=2048, vocab=32768, pattern="lLRAlLRA" * 2, scale_up=True))):
         REGISTRY[name] = layered_config(tukedra_config(**kw), name)
 

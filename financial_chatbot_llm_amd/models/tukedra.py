@@ -37,7 +37,7 @@ from .layered import Layer, LayeredDecoder
 from .mixers import DenseFF, TopSoftmaxRoutedFF
 
 
-def example_config(width: int = 160, vocab: int = 640, pattern: str = "lRaL", scale_up: bool = False, heads: int = 0,
+def example_config(width: int = 160, vocab: int = 768, pattern: str = "lRaL", scale_up: bool = False, heads: int = 0,
                    streams: int = 2) -> Dict:
     """A config.json-shaped dict for random-weight models (tests, benchmarks).  ``pattern``: one letter
     per layer -- l/L lightning, r/R retention, a/A attention; lower case with a dense feed-forward, upper

@@ -228,6 +228,21 @@ def test_first_tokens(device):
         close(run_whole(eng, f"r{n}", toks), oracle.forward(cfgd, sd, toks), torch.float32)
 
 
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("pattern", ["aA", "lR"])
+def test_single_mixer_kind_models(device, pattern):
+    """Only attention layers (no state slots at all) and only recurrent layers (no paged rows)."""
+    cfgd = small_config(pattern)
+    eng, sd = build(cfgd, device, torch.float32)
+    poison(eng)
+    assert (eng.state_slots is None) == (pattern == "aA")
+    toks = tokens(100, cfgd["vocab"], 17)
+    want = oracle.forward(cfgd, sd, toks)
+    got = [eng.replay_step([("r", toks[:70], list(range(70)))])]
+    got += [eng.replay_step([("r", toks[i:i + 1], [0])]) for i in range(70, 100)]
+    close(torch.cat(got), want, torch.float32)
+
+
 # ---------------------------------------------------------------------------------------------------
 # cache, state, batching
 # ---------------------------------------------------------------------------------------------------
