@@ -138,7 +138,8 @@ class TukedraModel(LayeredDecoder):
         self._sum_in = torch.ones(S, dtype=torch.float32, device=self.device)
 
     def logits(self, h: torch.Tensor) -> torch.Tensor:
-        return mx.logit_cap(F.linear(h, self.head), self.logit_scale, self.logit_softcap)
+        # scale and cap in f32: the head product is rounded once, not again after the tanh
+        return mx.logit_cap(F.linear(h, self.head).float(), self.logit_scale, self.logit_softcap)
 
     # -- forward -----------------------------------------------------------------------------------
     def forward(self, ids: torch.Tensor, positions: torch.Tensor, meta: AttentionMetadata, kv: HybridCache) -> torch.Tensor:
