@@ -186,6 +186,7 @@ def test_other_sizes(device, dtype):
     and sixth logits are often closer than the rounding of the router's input.)"""
     cfgd = small_config("ArLlaR" if dtype == torch.float32 else "arLlar", width=80, vocab=97, streams=4)
     cfgd["embedding"]["scale"] = 0.7
+    cfgd["norm"]["eps"] = 0.02               # large enough to show in every norm
     cfgd["logit_scale"], cfgd["logit_softcap"] = 1.7, 6.0
     L = cfgd["layers"]
     L[0]["mixer"].update(dim=40, vdim=40, heads=6, kv_heads=1, mask={"size": 70}, scale=0.31,
