@@ -28,6 +28,11 @@
 //   scans 16 tokens of one channel from zero, the sixteen partial maps S -> A S + B are folded through
 //   LDS, and the outputs are corrected by the true start state.  Steps of single rows (decode) take
 //   one fused launch instead.
+//
+// mx_mingru_scan: the minimal gated recurrent unit, S <- (1 - z) S + z c per channel with gates that read
+//   only the current token: z = sigmoid(zp + z_bias), u = xp + x_bias, c = u + 1/2 for u >= 0 and
+//   sigmoid(u) below; output S * silu(gp).  The same two launches (a gates pass that leaves 1 - z, z c
+//   and the SiLU branch in f32, then the recurrence kernel above) or one fused launch for single rows.
 #include "mx_common.h"
 
 namespace {
@@ -366,6 +371,48 @@ __global__ void lru_step_kernel(const float* __restrict__ u, const float* __rest
   }
 }
 
+__device__ __forceinline__ float mingru_candidate(float u) { return u >= 0.f ? u + 0.5f : mx_sigmoid(u); }
+
+// elementwise over [T, R]: ab[t, c] <- 1 - z, ab[t, R + c] <- z * candidate, gy[t, c] <- silu(g), all f32
+template <typename TI>
+__global__ void mingru_gates_kernel(const TI* __restrict__ zp, long sz, const TI* __restrict__ xp, long sx,
+                                    const TI* __restrict__ gp, long sg, const float* __restrict__ z_bias,
+                                    const float* __restrict__ x_bias, float* __restrict__ ab, float* __restrict__ gy,
+                                    long T, int R) {
+  const long total = T * R;
+  for (long e = blockIdx.x * (long)blockDim.x + threadIdx.x; e < total; e += (long)gridDim.x * blockDim.x) {
+    const long t = e / R;
+    const int c = (int)(e - t * R);
+    const float a = ldf(zp + t * sz + c) + (z_bias != nullptr ? z_bias[c] : 0.f);
+    const float u = ldf(xp + t * sx + c) + (x_bias != nullptr ? x_bias[c] : 0.f);
+    ab[t * 2 * R + c] = mx_sigmoid(-a);                              // 1 - sigmoid(a) without cancellation
+    ab[t * 2 * R + R + c] = mx_sigmoid(a) * mingru_candidate(u);
+    gy[e] = mx_silu(ldf(gp + t * sg + c));
+  }
+}
+
+// steps of single rows (decode): gates, recurrence and output in one launch, one thread per (row, channel)
+template <typename TI, typename TO>
+__global__ void mingru_step_kernel(const TI* __restrict__ zp, long sz, const TI* __restrict__ xp, long sx,
+                                   const TI* __restrict__ gp, long sg, const float* __restrict__ z_bias,
+                                   const float* __restrict__ x_bias, float* __restrict__ state,
+                                   const int* __restrict__ cu, const int* __restrict__ slot, const int* __restrict__ pos,
+                                   TO* __restrict__ out, int S, int R) {
+  const long total = (long)S * R;
+  for (long e = blockIdx.x * (long)blockDim.x + threadIdx.x; e < total; e += (long)gridDim.x * blockDim.x) {
+    const int s = (int)(e / R), c = (int)(e - (long)s * R);
+    const int sl = slot[s];
+    const long t = cu[s];
+    if (sl < 0 || cu[s + 1] <= t) continue;
+    const float a = ldf(zp + t * sz + c) + (z_bias != nullptr ? z_bias[c] : 0.f);
+    const float u = ldf(xp + t * sx + c) + (x_bias != nullptr ? x_bias[c] : 0.f);
+    const float prev = pos[t] == 0 ? 0.f : state[(long)sl * R + c];
+    const float Sn = mx_sigmoid(-a) * prev + mx_sigmoid(a) * mingru_candidate(u);
+    state[(long)sl * R + c] = Sn;
+    stf(out + t * R + c, Sn * mx_silu(ldf(gp + t * sg + c)));
+  }
+}
+
 template <typename TQ, int RPL, int LPC, int DELTA>
 int launch_matrix_scan(const void* q, long sq, const void* k, long sk, const void* v, long sv, const float* g, long sa,
                        const float* aux, float* state, const int* cu, const int* slot, const int* pos, float* out, int S,
@@ -487,5 +534,31 @@ MX_API int mx_lru_scan(float* u, float* z, int blocks, const float* r_bias, cons
                                                                  sy, y_bias, R));
   dim3 grid((R + LRU_CH - 1) / LRU_CH, S);
   MX_DISPATCH(dt_out, TO, lru_scan_kernel<TO><<<grid, 256, 0, st>>>(z, u, R / blocks, (long)T, state, cu, slot, pos, (TO*)out, R));
+  MX_RETURN_LAUNCH();
+}
+
+// zp, xp, gp [T, >= R] slices of type dt_in (row strides sz, sx, sg): pre-activations of the update gate, of
+// the candidate and of the output gate; z_bias, x_bias f32 [R] or null; ab f32 [T, 2R] and gy f32 [T, R]:
+// scratch (unused by single-row steps); state f32 [slots, R]; out [T, R] of type dt_out
+MX_API int mx_mingru_scan(const void* zp, long sz, const void* xp, long sx, const void* gp, long sg, int dt_in,
+                          const float* z_bias, const float* x_bias, float* ab, float* gy, float* state, const int* cu,
+                          const int* slot, const int* pos, void* out, int dt_out, int S, int R, int T, int max_len,
+                          hipStream_t st) {
+  if (S <= 0 || T <= 0) return 0;
+  if (R < 1) return (int)hipErrorInvalidValue;
+  if (max_len == 1) {
+    const long tot = (long)S * R;
+    const int g1 = (int)((tot + 255) / 256 < 8192 ? (tot + 255) / 256 : 8192);
+    MX_DISPATCH(dt_in, TI, MX_DISPATCH(dt_out, TO, mingru_step_kernel<TI, TO><<<g1, 256, 0, st>>>(
+        (const TI*)zp, sz, (const TI*)xp, sx, (const TI*)gp, sg, z_bias, x_bias, state, cu, slot, pos, (TO*)out, S, R)));
+    MX_RETURN_LAUNCH();
+  }
+  if (ab == nullptr || gy == nullptr) return (int)hipErrorInvalidValue;
+  const long total = (long)T * R;
+  const int gb = (int)((total + 255) / 256 < 8192 ? (total + 255) / 256 : 8192);
+  MX_DISPATCH(dt_in, TI, mingru_gates_kernel<TI><<<gb, 256, 0, st>>>((const TI*)zp, sz, (const TI*)xp, sx, (const TI*)gp, sg,
+                                                                     z_bias, x_bias, ab, gy, (long)T, R));
+  dim3 grid((R + LRU_CH - 1) / LRU_CH, S);
+  MX_DISPATCH(dt_out, TO, lru_scan_kernel<TO><<<grid, 256, 0, st>>>(ab, gy, R, (long)T, state, cu, slot, pos, (TO*)out, R));
   MX_RETURN_LAUNCH();
 }

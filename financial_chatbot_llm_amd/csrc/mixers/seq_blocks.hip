@@ -3,7 +3,7 @@
 //   * layer norm on a sublayer's OUTPUT fused with the residual add and the rounding of the next
 //     GEMM input:  x <- x + LN(m) * w,  m = a  or  m = (RMSnorm(a) * wa + RMSnorm(b) * wb) / 2
 //     (two mixers side by side);  without a: out = LN(x) * w (the model's last norm);
-//   * gated activations act(s * gate) * (s * up) with an optional scale per row;
+//   * gated activations act(s * gate) * (s * up) with an optional scale per row (or act alone);
 //   * top-k routing on independent sigmoid (or softmax) scores;
 //   * per-head RMS norm with a weight shared by the heads, times an activated gate.
 #include "mx_common.h"
@@ -117,7 +117,8 @@ __global__ void glu_act_kernel(const T* __restrict__ gate, long sg, const T* __r
     const long t = i / n;
     const int c = (int)(i - t * n);
     const float s = row_scale != nullptr ? row_scale[t] : 1.0f;
-    stf(out + t * so + c, mx_act(s * ldf(gate + t * sg + c), act) * (s * ldf(up + t * su + c)));
+    const float g = mx_act(s * ldf(gate + t * sg + c), act);
+    stf(out + t * so + c, up != nullptr ? g * (s * ldf(up + t * su + c)) : g);
   }
 }
 
@@ -230,7 +231,7 @@ MX_API int mx_post_norm(float* x, const void* a, long sa, const float* wa, const
   MX_RETURN_LAUNCH();
 }
 
-// act: 1 SiLU, 2 tanh-form GeLU
+// act: 1 SiLU, 2 tanh-form GeLU; up null: the activation alone
 MX_API int mx_glu_act(const void* gate, long sg, const void* up, long su, const float* row_scale, int act, void* out,
                       long so, int dt, int T, int n, hipStream_t st) {
   const long total = (long)T * n;

@@ -2,6 +2,8 @@
 //   * embedding gather into an f32 stream;
 //   * parallel-block residual update fused with the next RMS norm:
 //         x <- x + mult * (a + b);  y = x / sqrt(mean(x^2) + eps) * w
+//     optionally with a weight per sublayer output and a sigmoid gate per element on the update:
+//         x <- x + sigmoid(gate + gate_bias) * (mult_a * a + mult_b * b)
 //   * RMS norm of a strided row slice (latent norms), optionally in equal groups and with a SiLU
 //     gate applied first (the state-space mixer's output norm);
 //   * activations: relu^2, and the clamped gated unit g * sigmoid(alpha g) * (u + 1);
@@ -21,10 +23,12 @@ __global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ 
   for (int i = threadIdx.x; i < W; i += blockDim.x) out[(long)t * W + i] = ldf(row + i);
 }
 
-// one block per row.  a / b: the two sublayer outputs of a parallel block (either may be null).
+// one block per row.  a / b: the two sublayer outputs of a parallel block (either may be null);
+// gate (may be null): pre-activations of a sigmoid gate on the update, gate_bias f32 [W] or null.
 template <typename TA, typename TO>
 __global__ void residual_norm_kernel(float* __restrict__ x, const TA* __restrict__ a, long sa,
-                                     const TA* __restrict__ b, long sb, float mult,
+                                     const TA* __restrict__ b, long sb, float mult, float mult_b,
+                                     const TA* __restrict__ gate, long sg, const float* __restrict__ gate_bias,
                                      const float* __restrict__ w, float eps, TO* __restrict__ out, int W) {
   __shared__ float scratch[16];
   const long t = blockIdx.x;
@@ -33,10 +37,17 @@ __global__ void residual_norm_kernel(float* __restrict__ x, const TA* __restrict
   for (int i = threadIdx.x; i < W; i += blockDim.x) {
     float v = xr[i];
     if (a != nullptr || b != nullptr) {
-      float s = 0.f;
-      if (a != nullptr) s += ldf(a + t * sa + i);
-      if (b != nullptr) s += ldf(b + t * sb + i);
-      v = v + mult * s;
+      float s;
+      if (mult == mult_b) {
+        s = 0.f;
+        if (a != nullptr) s += ldf(a + t * sa + i);
+        if (b != nullptr) s += ldf(b + t * sb + i);
+        s *= mult;
+      } else {
+        s = (a != nullptr ? mult * ldf(a + t * sa + i) : 0.f) + (b != nullptr ? mult_b * ldf(b + t * sb + i) : 0.f);
+      }
+      if (gate != nullptr) s *= mx_sigmoid(ldf(gate + t * sg + i) + (gate_bias != nullptr ? gate_bias[i] : 0.f));
+      v = v + s;
       xr[i] = v;
     }
     ss += v * v;
@@ -173,13 +184,15 @@ MX_API int mx_embed(const int* ids, const void* table, int dt, float* out, int T
   MX_RETURN_LAUNCH();
 }
 
-// x [T, W] f32 (updated in place when a or b is given); out (may be null: update only) of type dt_out
+// x [T, W] f32 (updated in place when a or b is given); out (may be null: update only) of type dt_out;
+// a, b and gate (a [T, >= W] slice, or null) of type dt_ab; mult weighs a, mult_b weighs b
 MX_API int mx_residual_norm(float* x, const void* a, long sa, const void* b, long sb, int dt_ab, float mult,
-                            const float* w, float eps, void* out, int dt_out, int T, int W, hipStream_t st) {
+                            float mult_b, const void* gate, long sg, const float* gate_bias, const float* w, float eps,
+                            void* out, int dt_out, int T, int W, hipStream_t st) {
   if (T <= 0) return 0;
   const int nt = W >= 1024 ? 512 : 256;
   MX_DISPATCH(dt_ab, TA, MX_DISPATCH(dt_out, TO, residual_norm_kernel<TA, TO><<<T, nt, 0, st>>>(
-      x, (const TA*)a, sa, (const TA*)b, sb, mult, w, eps, (TO*)out, W)));
+      x, (const TA*)a, sa, (const TA*)b, sb, mult, mult_b, (const TA*)gate, sg, gate_bias, w, eps, (TO*)out, W)));
   MX_RETURN_LAUNCH();
 }
 

@@ -90,7 +90,8 @@ __global__ void __launch_bounds__(RH_WAVES * 64)
 rope_heads_kernel(const TI* __restrict__ q, long sq, int Hq, const TI* __restrict__ k, long sk, int Hk, int D, int rot,
                   int half, const float* __restrict__ freq, float mscale, const int* __restrict__ pos, int norm,
                   float eps, float qscale, float kscale, TQ* __restrict__ qout, TK* __restrict__ kout, long sko,
-                  const int* __restrict__ slots, const TI* __restrict__ v, long sv, int nv) {
+                  const int* __restrict__ slots, const TI* __restrict__ v, long sv, int nv,
+                  const TI* __restrict__ vmix, long svm, float lam) {
   extern __shared__ float buf[];             // [RH_WAVES][D]
   const long t = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -134,7 +135,11 @@ rope_heads_kernel(const TI* __restrict__ q, long sq, int Hq, const TI* __restric
   }
   if (v != nullptr && krow >= 0) {
     TK* dst = kout + krow * sko + (long)Hk * D;
-    for (int i = threadIdx.x; i < nv; i += blockDim.x) stf(dst + i, ldf(v + t * sv + i));
+    if (vmix != nullptr)       // blended in f32, rounded once into the cache row
+      for (int i = threadIdx.x; i < nv; i += blockDim.x)
+        stf(dst + i, (1.0f - lam) * ldf(v + t * sv + i) + lam * ldf(vmix + t * svm + i));
+    else
+      for (int i = threadIdx.x; i < nv; i += blockDim.x) stf(dst + i, ldf(v + t * sv + i));
   }
 }
 
@@ -184,18 +189,21 @@ MX_API int mx_hyper_mix(float* x, const void* y, long sy, int dt_y, const float*
 // q [T, Hq*D], k [T, Hk*D] slices of type dt_in (row strides sq, sk); freq f32 [rot / 2] (rot = 0: no
 // rotation); half != 0: pairs (i, i + rot/2), else (2i, 2i+1); qout [T, Hq*D] contiguous of type dt_q; kout
 // rows of stride sko and type dt_k, row slots[t] (slots null: row t; a negative slot: no write); v (may be
-// null): nv raw values of type dt_in copied behind the keys of the same row
+// null): nv raw values of type dt_in copied behind the keys of the same row -- with vmix (same shape and
+// type, row stride svm) as (1 - lam) v + lam vmix
 MX_API int mx_rope_heads(const void* q, long sq, int Hq, const void* k, long sk, int Hk, int dt_in, int D, int rot,
                          int half, const float* freq, float mscale, const int* pos, int norm, float eps, float qscale,
                          float kscale, void* qout, int dt_q, void* kout, long sko, int dt_k, const int* slots,
-                         const void* v, long sv, int nv, int T, hipStream_t st) {
+                         const void* v, long sv, int nv, const void* vmix, long svm, float lam, int T,
+                         hipStream_t st) {
   if (T <= 0) return 0;
   if (D < 1 || rot < 0 || rot > D || (rot & 1) || (rot > 0 && freq == nullptr) || D > 4096)
     return (int)hipErrorInvalidValue;
   const size_t lds = (size_t)RH_WAVES * D * sizeof(float);
   MX_DISPATCH(dt_in, TI, MX_DISPATCH(dt_q, TQ, MX_DISPATCH(dt_k, TK, rope_heads_kernel<TI, TQ, TK>
       <<<T, RH_WAVES * 64, lds, st>>>((const TI*)q, sq, Hq, (const TI*)k, sk, Hk, D, rot, half, freq, mscale, pos, norm,
-                                      eps, qscale, kscale, (TQ*)qout, (TK*)kout, sko, slots, (const TI*)v, sv, nv))));
+                                      eps, qscale, kscale, (TQ*)qout, (TK*)kout, sko, slots, (const TI*)v, sv, nv,
+                                      (const TI*)vmix, svm, lam))));
   MX_RETURN_LAUNCH();
 }
 

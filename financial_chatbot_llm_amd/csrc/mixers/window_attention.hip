@@ -6,7 +6,12 @@
 // positions (floor(j / window) == floor(p / window), blocks counted from position 0 of the sequence);
 // score = q . k * scale; softmax and accumulation in f32; the head's output is multiplied by
 // sigmoid(gate[t, h]) when a gate is given.  Rotation and norms of q and k happen before (the cache holds
-// finished keys).
+// finished keys).  Two further forms of the same walk:
+//   * kept first tokens (attention sinks): with keep > 0 the keys j < keep stay visible to every later
+//     query whatever the window (at their true positions); the tiles that hold them are walked before the
+//     window's own tiles;
+//   * sigmoid weights: with a per-head bias array the weight of a visible key is
+//     sigmoid(score + head_bias[h]) and the weights are NOT normalised over the keys (no softmax).
 //
 //   mx_qk_norm_write   RMS norm over the WHOLE query projection and over the whole key projection
 //                      (all heads at once, plain weights), cache write of [normed k | v].
@@ -23,6 +28,12 @@ constexpr int PAGE = 64;            // tokens per cache page
 // first key the query at position p sees: a sliding window of `window` keys, or the start of p's block
 __device__ __forceinline__ int first_key(int p, int window, int chunked) {
   return chunked ? (p / window) * window : max(0, p - window + 1);
+}
+
+// The tiles a block walks: `nsink` tiles from key 0 that hold kept first tokens and lie wholly before
+// the window's first tile, then the tiles first_tile .. last_tile.  Walk index -> first key of the tile.
+__device__ __forceinline__ int walk_k0(int ti, int nsink, int first_tile, int KT) {
+  return (ti < nsink ? ti : first_tile + ti - nsink) * KT;
 }
 
 // one block per token
@@ -74,8 +85,8 @@ template <typename T>
 __global__ void __launch_bounds__(WA_WAVES * 64)
 window_attend_kernel(const T* __restrict__ q, long sq, const T* __restrict__ cache, const int* __restrict__ cu,
                      const int* __restrict__ pos, const int* __restrict__ bt, int btw, const T* __restrict__ gate,
-                     long sgate, int window, int chunked, float scale, T* __restrict__ out, int H, int G, int D, int P,
-                     int QT, int HB, int KT, int ldk, int ldv) {
+                     long sgate, int window, int chunked, int keep, const float* __restrict__ hbias, float scale,
+                     T* __restrict__ out, int H, int G, int D, int P, int QT, int HB, int KT, int ldk, int ldv) {
   extern __shared__ __align__(16) unsigned char smem[];
   T* ktile = reinterpret_cast<T*>(smem);                                  // [KT][ldk]
   T* vtile = ktile + (size_t)KT * ldk;                                    // [KT][ldv]
@@ -110,7 +121,11 @@ window_attend_kernel(const T* __restrict__ q, long sq, const T* __restrict__ cac
     for (int c = 0; c < WA_CPL; ++c) acc[i][c] = 0.f;
   }
 
-  for (int k0 = (lo / KT) * KT; k0 <= p_last; k0 += KT) {
+  const int first_tile = lo / KT;
+  const int nsink = min((keep + KT - 1) / KT, first_tile);
+  const int ntiles = nsink + p_last / KT - first_tile + 1;
+  for (int ti = 0; ti < ntiles; ++ti) {
+    const int k0 = walk_k0(ti, nsink, first_tile, KT);
     __syncthreads();                       // previous tile fully consumed
     const int rows = min(KT, p_last + 1 - k0);   // only these rows of the tile are staged (and read)
     {
@@ -134,7 +149,7 @@ window_attend_kernel(const T* __restrict__ q, long sq, const T* __restrict__ cac
       const int h = h0 + hh;
       const int p = pos[row];
       const int j = k0 + lane;
-      const bool vis = lane < rows && j <= p && j >= first_key(p, window, chunked);
+      const bool vis = lane < rows && j <= p && (j >= first_key(p, window, chunked) || j < keep);
       if (__ballot(vis) == 0ull) continue;                // no visible key of this tile
       {
         const T* qh = q + row * sq + (long)h * D;
@@ -148,12 +163,17 @@ window_attend_kernel(const T* __restrict__ q, long sq, const T* __restrict__ cac
         for (int d = 0; d < D; ++d) a += myq[d] * ldf(kr + d);
         sc = a * scale;
       }
-      const float mt = mx_wave_max(sc);
-      const float mn = fmaxf(m[ii], mt);
-      const float corr = expf(m[ii] - mn);                 // exp(-inf) = 0 on the first tile
-      const float pj = vis ? expf(sc - mn) : 0.f;
-      l[ii] = l[ii] * corr + mx_wave_sum(pj);
-      m[ii] = mn;
+      float corr = 1.f, pj;
+      if (hbias != nullptr) {                              // independent sigmoid weights, no running statistics
+        pj = vis ? mx_sigmoid(sc + hbias[h]) : 0.f;
+      } else {
+        const float mt = mx_wave_max(sc);
+        const float mn = fmaxf(m[ii], mt);
+        corr = expf(m[ii] - mn);                           // exp(-inf) = 0 on the first tile
+        pj = vis ? expf(sc - mn) : 0.f;
+        l[ii] = l[ii] * corr + mx_wave_sum(pj);
+        m[ii] = mn;
+      }
       myp[lane] = pj;
       // one wave writes and reads myq / myp: its LDS accesses complete in program order
       __builtin_amdgcn_wave_barrier();
@@ -176,7 +196,7 @@ window_attend_kernel(const T* __restrict__ q, long sq, const T* __restrict__ cac
     const int tq = item / nh, hh = item - tq * nh;
     const long row = r0 + t0 + tq;
     const int h = h0 + hh;
-    float gs = 1.0f / l[ii];
+    float gs = hbias != nullptr ? 1.0f : 1.0f / l[ii];
     if (gate != nullptr) gs *= mx_sigmoid(ldf(gate + row * sgate + h));
 #pragma unroll
     for (int c = 0; c < WA_CPL; ++c) {
@@ -209,9 +229,9 @@ template <int KSM, int NTM>         // up to 32*KSM key dims, 16*NTM value dims
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
 window_attend_mfma_kernel(const bf16* __restrict__ q, long sq, const bf16* __restrict__ cache,
                           const int* __restrict__ cu, const int* __restrict__ pos, const int* __restrict__ bt, int btw,
-                          const bf16* __restrict__ gate, long sgate, int window, int chunked, float scale,
-                          bf16* __restrict__ out, int H, int G, int D, int P, int QT, int HB, int nsplit,
-                          float* __restrict__ ws) {
+                          const bf16* __restrict__ gate, long sgate, int window, int chunked, int keep,
+                          const float* __restrict__ hbias, float scale, bf16* __restrict__ out, int H, int G, int D,
+                          int P, int QT, int HB, int nsplit, float* __restrict__ ws) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int KS = (D + 31) / 32, NT = (P + 15) / 16;
   const int ldk = KS * 32 + 8;
@@ -244,6 +264,8 @@ window_attend_mfma_kernel(const bf16* __restrict__ q, long sq, const bf16* __res
   const int pq = qok ? pos[row] : -1;
   const int pq_lo = qok ? first_key(pq, window, chunked) : 0;
   const bool wave_live = 16 * wave < nq * nh;
+  const bool sigm = hbias != nullptr;
+  const float hb = (sigm && qok) ? hbias[h] : 0.f;
 
   bf16x8 qf[KSM];
 #pragma unroll
@@ -266,12 +288,13 @@ window_attend_mfma_kernel(const bf16* __restrict__ q, long sq, const bf16* __res
     for (int e = threadIdx.x; e < words; e += 256) z[e] = 0u;
   }
 
-  int k_begin = (lo / MKT) * MKT, k_end = p_last;     // first tile start, last key
+  const int first_tile = lo / MKT;
+  const int nsink = min((keep + MKT - 1) / MKT, first_tile);
+  int t_begin = 0, t_end = nsink + p_last / MKT - first_tile;     // walk indices, inclusive
   if (nsplit > 1) {
-    const int tiles = (p_last - k_begin) / MKT + 1;
-    const int per = (tiles + nsplit - 1) / nsplit;
-    k_begin += split * per * MKT;
-    k_end = min(p_last, k_begin + per * MKT - 1);
+    const int per = (t_end + nsplit) / nsplit;                    // ceil((t_end + 1) / nsplit)
+    t_begin = split * per;
+    t_end = min(t_end, t_begin + per - 1);
   }
   // staging, 16-byte path (D, P multiples of 8): a work item is a pair of keys x 8 dims of the key
   // part or of the value part -- two row loads; key pieces go to the key tile as two 16-byte stores,
@@ -318,8 +341,9 @@ window_attend_mfma_kernel(const bf16* __restrict__ q, long sq, const bf16* __res
       }
     }
   };
-  if (v16 && k_begin <= k_end) load_tile(k_begin);
-  for (int k0 = k_begin; k0 <= k_end; k0 += MKT) {
+  if (v16 && t_begin <= t_end) load_tile(walk_k0(t_begin, nsink, first_tile, MKT));
+  for (int ti = t_begin; ti <= t_end; ++ti) {
+    const int k0 = walk_k0(ti, nsink, first_tile, MKT);
     __syncthreads();
     const int rows = min(MKT, p_last + 1 - k0);
     if (v16) {
@@ -336,7 +360,7 @@ window_attend_mfma_kernel(const bf16* __restrict__ q, long sq, const bf16* __res
       }
     }
     __syncthreads();
-    if (v16 && k0 + MKT <= k_end) load_tile(k0 + MKT);
+    if (v16 && ti < t_end) load_tile(walk_k0(ti + 1, nsink, first_tile, MKT));
     if (!wave_live) continue;
     // S^T for the two 16-key halves
     f32x4 st[2];
@@ -352,7 +376,7 @@ window_attend_mfma_kernel(const bf16* __restrict__ q, long sq, const bf16* __res
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int j = k0 + 16 * kh + 4 * g + i;
-        const bool vis = j <= pq && j >= pq_lo;
+        const bool vis = j <= pq && (j >= pq_lo || j < keep);
         sc[kh][i] = vis ? st[kh][i] * scale : -INFINITY;
         tmax = fmaxf(tmax, sc[kh][i]);
       }
@@ -360,7 +384,7 @@ window_attend_mfma_kernel(const bf16* __restrict__ q, long sq, const bf16* __res
     tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
     const float mn = fmaxf(m, tmax);
-    const float corr = (m == -INFINITY) ? 0.f : expf(m - mn);
+    const float corr = sigm ? 1.f : ((m == -INFINITY) ? 0.f : expf(m - mn));
     // the f32 weight enters the value product as two bf16 terms, p = hi + lo (16 mantissa bits: far
     // below the rounding of the bf16 values it multiplies), both accumulated in f32
     bf16x8 pb, pl;
@@ -369,7 +393,7 @@ window_attend_mfma_kernel(const bf16* __restrict__ q, long sq, const bf16* __res
     for (int kh = 0; kh < 2; ++kh)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float p = sc[kh][i] == -INFINITY ? 0.f : expf(sc[kh][i] - mn);
+        const float p = sc[kh][i] == -INFINITY ? 0.f : (sigm ? mx_sigmoid(sc[kh][i] + hb) : expf(sc[kh][i] - mn));
         psum += p;
         const bf16 hi = (bf16)p;
         pb[4 * kh + i] = hi;
@@ -413,7 +437,7 @@ window_attend_mfma_kernel(const bf16* __restrict__ q, long sq, const bf16* __res
     }
     return;
   }
-  float gsc = 1.0f / l;
+  float gsc = sigm ? 1.0f : 1.0f / l;
   if (gate != nullptr) gsc *= mx_sigmoid((float)gate[row * sgate + h]);
   bf16* dst = out + (row * H + h) * P;
 #pragma unroll
@@ -429,11 +453,21 @@ window_attend_mfma_kernel(const bf16* __restrict__ q, long sq, const bf16* __res
 }
 
 // grid (rows, H): combine the nsplit parts of one (row, head)
+// (sigm: the parts are plain sums of independently weighted values)
 __global__ void window_merge_kernel(const float* __restrict__ ws, const bf16* __restrict__ gate, long sgate,
-                                    bf16* __restrict__ out, int H, int P, int nsplit) {
+                                    bf16* __restrict__ out, int H, int P, int nsplit, int sigm) {
   const long row = blockIdx.x;
   const int h = blockIdx.y;
   const float* w = ws + (row * H + h) * nsplit * (long)(P + 2);
+  if (sigm) {
+    const float gs = gate != nullptr ? mx_sigmoid((float)gate[row * sgate + h]) : 1.0f;
+    for (int r = threadIdx.x; r < P; r += blockDim.x) {
+      float a = 0.f;
+      for (int i = 0; i < nsplit; ++i) a += w[i * (P + 2) + r];
+      out[(row * H + h) * P + r] = (bf16)(a * gs);
+    }
+    return;
+  }
   float M = -INFINITY;
   for (int i = 0; i < nsplit; ++i) M = fmaxf(M, w[i * (P + 2) + P]);
   float L = 0.f;
@@ -479,14 +513,16 @@ MX_API int mx_qk_norm_write(const void* q, long sq, const void* k, long sk, cons
 // q [T, H*D] (row stride sq), out [T, H*P] contiguous; cu [S+1] row bounds of the segments, pos [T]
 // positions, bt [S, btw] page tables; gate [T, >= H] slice (row stride sgate) or null.
 // chunked != 0: `window` is the block size of the chunked mask instead of a sliding window's length.
+// keep > 0: the first `keep` keys of the sequence stay visible beyond the window.  head_bias (f32 [H], or
+// null): sigmoid weights sigmoid(score + head_bias[h]) without normalisation instead of a softmax.
 // nsplit > 1 with a workspace ws (f32 [T, H, nsplit, P + 2]) and single-row segments: the key range of
 // each row is walked by nsplit blocks and merged (bf16 matrix-core form only; ignored otherwise).
 MX_API int mx_window_attend(const void* q, long sq, const void* cache, const int* cu, const int* pos, const int* bt,
-                            int btw, const void* gate, long sgate, int window, int chunked, float scale, void* out,
-                            int dt, int S, int max_len, int H, int G, int D, int P, int nsplit, float* ws,
-                            hipStream_t st) {
+                            int btw, const void* gate, long sgate, int window, int chunked, int keep,
+                            const float* head_bias, float scale, void* out, int dt, int S, int max_len, int H, int G,
+                            int D, int P, int nsplit, float* ws, hipStream_t st) {
   if (S <= 0 || max_len <= 0) return 0;
-  if (P > 64 * WA_CPL || G < 1 || H % G || window < 1) return (int)hipErrorInvalidValue;
+  if (P > 64 * WA_CPL || G < 1 || H % G || window < 1 || keep < 0) return (int)hipErrorInvalidValue;
   const int rep = H / G;
   if (dt == 0 && D <= 256 && P <= 256 && wa_use_mfma()) {
     // matrix-core form: 64 (row, head) pairs of one key/value head per block
@@ -498,15 +534,16 @@ MX_API int mx_window_attend(const void* q, long sq, const void* cache, const int
     dim3 grid(nsplit > 1 ? nsplit : (max_len + QT - 1) / QT, G * ((rep + HB - 1) / HB), S);
     if (D <= 128 && P <= 128)
       window_attend_mfma_kernel<4, 8><<<grid, 256, lds, st>>>(
-          (const bf16*)q, sq, (const bf16*)cache, cu, pos, bt, btw, (const bf16*)gate, sgate, window, chunked, scale,
-          (bf16*)out, H, G, D, P, QT, HB, nsplit, ws);
+          (const bf16*)q, sq, (const bf16*)cache, cu, pos, bt, btw, (const bf16*)gate, sgate, window, chunked, keep,
+          head_bias, scale, (bf16*)out, H, G, D, P, QT, HB, nsplit, ws);
     else
       window_attend_mfma_kernel<8, 16><<<grid, 256, lds, st>>>(
-          (const bf16*)q, sq, (const bf16*)cache, cu, pos, bt, btw, (const bf16*)gate, sgate, window, chunked, scale,
-          (bf16*)out, H, G, D, P, QT, HB, nsplit, ws);
+          (const bf16*)q, sq, (const bf16*)cache, cu, pos, bt, btw, (const bf16*)gate, sgate, window, chunked, keep,
+          head_bias, scale, (bf16*)out, H, G, D, P, QT, HB, nsplit, ws);
     if (nsplit > 1) {
       dim3 g2(S, H);           // single-row segments: row index == segment index
-      window_merge_kernel<<<g2, P >= 128 ? 128 : 64, 0, st>>>(ws, (const bf16*)gate, sgate, (bf16*)out, H, P, nsplit);
+      window_merge_kernel<<<g2, P >= 128 ? 128 : 64, 0, st>>>(ws, (const bf16*)gate, sgate, (bf16*)out, H, P, nsplit,
+                                                              head_bias != nullptr ? 1 : 0);
     }
     MX_RETURN_LAUNCH();
   }
@@ -530,7 +567,7 @@ MX_API int mx_window_attend(const void* q, long sq, const void* cache, const int
   if (lds > 64 * 1024) return (int)hipErrorInvalidValue;
   dim3 grid((max_len + QT - 1) / QT, G * ((rep + HB - 1) / HB), S);
   MX_DISPATCH(dt, TT, window_attend_kernel<TT><<<grid, WA_WAVES * 64, lds, st>>>(
-      (const TT*)q, sq, (const TT*)cache, cu, pos, bt, btw, (const TT*)gate, sgate, window, chunked, scale, (TT*)out, H, G,
-      D, P, QT, HB, KT, ldk, ldv));
+      (const TT*)q, sq, (const TT*)cache, cu, pos, bt, btw, (const TT*)gate, sgate, window, chunked, keep, head_bias,
+      scale, (TT*)out, H, G, D, P, QT, HB, KT, ldk, ldv));
   MX_RETURN_LAUNCH();
 }

@@ -1,4 +1,4 @@
-"""Model families: Llama-3 (8B/70B), Mixtral-8x7B MoE, BERT/bge encoder, and the layered decoders Gezavik, Sigudra and Tukedra."""
+"""Model families: Llama-3 (8B/70B), Mixtral-8x7B MoE, BERT/bge encoder, and the layered decoders Gezavik, Sigudra, Tukedra and Purozen."""
 from __future__ import annotations
 
 from .configs import LAYERED_ARCHS, REGISTRY, ModelConfig, get_model_config
@@ -42,9 +42,10 @@ def _build_layered(cfg, engine_cfg, device, seed: int):
 
     from .gezavik import GezavikModel
     from .sigudra import SigudraModel
+    from .purozen import PurozenModel
     from .tukedra import TukedraModel
     from .weights import read_safetensors
-    cls = {"gezavik": GezavikModel, "sigudra": SigudraModel, "tukedra": TukedraModel}[cfg.arch]
+    cls = {"gezavik": GezavikModel, "sigudra": SigudraModel, "tukedra": TukedraModel, "purozen": PurozenModel}[cfg.arch]
     if getattr(engine_cfg, "tp_size", 1) > 1:
         raise ValueError(f"{cfg.name}: tensor parallelism is not implemented for layered decoders")
     dtype = str(getattr(engine_cfg, "dtype", "bf16")).lower()

@@ -15,7 +15,7 @@ from typing import Dict, Optional
 @dataclass(frozen=True)
 class ModelConfig:
     name: str
-    arch: str                       # "llama" | "mixtral" | "bert" | "gezavik" | "sigudra" | "tukedra"
+    arch: str                       # "llama" | "mixtral" | "bert" | "gezavik" | "sigudra" | "tukedra" | "purozen"
     vocab_size: int
     hidden_size: int
     num_layers: int
@@ -85,6 +85,7 @@ def _register_layered() -> None:
     from .gezavik import example_config
     from .sigudra import example_config as sigudra_config
     from .tukedra import example_config as tukedra_config
+    from .purozen import example_config as purozen_config
     for name, kw in (("gezavik-tiny", dict(width=192, vocab=1024, heads=3, pattern="amAm")),
                      ("gezavik-1b", dict(width=2048, vocab=32768, heads=16, pattern="aMmAmMaM" * 2, scale_up=True))):
         REGISTRY[name] = layered_config(example_config(**kw), name)
@@ -94,10 +95,13 @@ def _register_layered() -> None:
     for name, kw in (("tukedra-tiny", dict(width=160, vocab=768, pattern="lRaL")),
                      ("tukedra-1b", dict(width=2048, vocab=32768, pattern="lLRAlLRA" * 2, scale_up=True))):
         REGISTRY[name] = layered_config(tukedra_config(**kw), name)
+    for name, kw in (("purozen-tiny", dict(width=160, vocab=896, pattern="paAl")),
+                     ("purozen-1b", dict(width=2048, vocab=32768, pattern="paalpaal" * 2, scale_up=True))):
+        REGISTRY[name] = layered_config(purozen_config(**kw), name)
 
 
 def get_model_config(name: str) -> ModelConfig:
-    if name.startswith(("gezavik-", "sigudra-", "tukedra-")) and name not in REGISTRY:
+    if name.startswith(("gezavik-", "sigudra-", "tukedra-", "purozen-")) and name not in REGISTRY:
         _register_layered()
     if name in REGISTRY:
         return REGISTRY[name]
@@ -132,7 +136,7 @@ def from_hf(path: str, name: Optional[str] = None) -> ModelConfig:
         top_k_experts=c.get("num_experts_per_tok", 0), bos_token_id=c.get("bos_token_id", 1), eos_token_ids=eos)
 
 
-LAYERED_ARCHS = ("gezavik", "sigudra", "tukedra")
+LAYERED_ARCHS = ("gezavik", "sigudra", "tukedra", "purozen")
 
 
 def layered_config(c: Dict, name: Optional[str] = None) -> ModelConfig:
@@ -148,7 +152,7 @@ def layered_config(c: Dict, name: Optional[str] = None) -> ModelConfig:
     win = next((l["mixer"]["left"] for l in layers if "left" in l["mixer"]), None)
     win = win or next((l["mixer"] for l in layers if l.get("type") == "attention"), None)
     heads = att["heads"] if att else (win["heads"] if win else 1)
-    hd = (att["dim"] + att["rot_dim"]) if att else (win["dim"] if win else c["width"])
+    hd = (att["dim"] + att.get("rot_dim", 0)) if att else (win["dim"] if win else c["width"])
     ffs = [l["mlp"]["ff"] for l in layers if l.get("mlp") and l["mlp"].get("kind") == "dense"]
     return ModelConfig(name or arch, arch, c["vocab"], c["width"], len(layers), heads, 1, hd, max(ffs, default=0),
                        max_position=1 << 24, norm_eps=float(c["norm"]["eps"]), bos_token_id=0, eos_token_ids=(),

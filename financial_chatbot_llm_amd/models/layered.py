@@ -1,4 +1,4 @@
-"""Common part of the layered decoders (:mod:`.gezavik`, :mod:`.sigudra`, :mod:`.tukedra`): a ``config.json`` lists the
+"""Common part of the layered decoders (:mod:`.gezavik`, :mod:`.sigudra`, :mod:`.tukedra`, :mod:`.purozen`): a ``config.json`` lists the
 layers, each with one sequence mixer of :mod:`.mixers` and optionally one feed-forward; the residual
 stream is f32 whatever the activation dtype; the checkpoint is the model directory itself (tensors
 ``embed``, ``l<i>.<norm>``, ``l<i>.mix.<name>``, ``l<i>.mlp.<name>``, ``final.norm``, ``head``; linear
@@ -28,10 +28,11 @@ class Layer:
     def __init__(self, i: int, spec: Dict, width: int, eps: float, mixer_types=None):
         self.prefix = f"l{i}"
         kind = spec["type"]
-        if kind not in MIXERS or (mixer_types is not None and kind not in mixer_types):
-            known = sorted(mixer_types if mixer_types is not None else MIXERS)
-            raise ValueError(f"layer {i}: unknown mixer type {kind!r}; known: {known}")
-        self.mixer = MIXERS[kind](spec["mixer"], width, eps)
+        # a design names its mixer types: a tuple of registry names, or {the design's own name: registry name}
+        names = mixer_types if isinstance(mixer_types, dict) else {k: k for k in (mixer_types or MIXERS)}
+        if kind not in names or names[kind] not in MIXERS:
+            raise ValueError(f"layer {i}: unknown mixer type {kind!r}; known: {sorted(names)}")
+        self.mixer = MIXERS[names[kind]](spec["mixer"], width, eps)
         self.ff = None
         self.w_in: Optional[torch.Tensor] = None
         self.norm1: Optional[torch.Tensor] = None
@@ -52,6 +53,7 @@ class LayeredDecoder:
     tp_size = 1
     tp_rank = 0
     slot_arrays: Dict = {}       # per-slot records of the model as a whole: {name: (dtype, shape)}
+    tied_head = False            # the vocabulary projection is the embedding table (no ``head`` tensor)
 
     def __init__(self, cfg: ModelConfig, device="cuda", dtype=torch.bfloat16):
         if cfg.arch != self.arch or not cfg.layers:
@@ -81,7 +83,9 @@ class LayeredDecoder:
     def full_shapes(self) -> Dict[str, tuple]:
         """Checkpoint names and shapes; a ``None`` entry is a size only the tensor itself gives."""
         c = self.cfg
-        s = {"embed": (c.vocab_size, c.hidden_size), "final.norm": (c.hidden_size,), "head": (c.vocab_size, c.hidden_size)}
+        s = {"embed": (c.vocab_size, c.hidden_size), "final.norm": (c.hidden_size,)}
+        if not self.tied_head:
+            s["head"] = (c.vocab_size, c.hidden_size)
         s.update(self.extra_shapes())
         for l in self.layers:
             for n in l.norms():
@@ -115,6 +119,10 @@ class LayeredDecoder:
             return 1.0 + 0.2 * randn()
         if leaf == "correction":
             return 0.05 * randn()
+        if leaf == "vmix":         # blend weight of the first layer's values
+            return 0.2 + 0.6 * rand()
+        if leaf == "pb":           # sigmoid attention: weights start small
+            return -2.0 + 0.5 * randn()
         if name.endswith("a2.b"):  # decay gates biased toward slow decay
             return 2.0 + 0.5 * randn()
         if leaf == "b" and (len(shape) == 1 or name.endswith(("ra.b", "ri.b"))):     # biases
@@ -146,7 +154,7 @@ class LayeredDecoder:
         dev, dt = self.device, self.dtype
         get = lambda n: sd[n].to(dev)  # noqa: E731
         self.embed = get("embed").to(dt).contiguous()
-        self.head = get("head").to(dt).contiguous()
+        self.head = self.embed if self.tied_head else get("head").to(dt).contiguous()
         self.final_norm = get("final.norm").float().contiguous()
         self.load_extra(get)
         for l in self.layers:
@@ -154,7 +162,7 @@ class LayeredDecoder:
         return self
 
     def weight_tensors(self):
-        ts = [self.embed, self.head]
+        ts = [self.embed] if self.tied_head else [self.embed, self.head]
         for l in self.layers:
             ts += [t for t in (l.w_in, getattr(l, "w_ff", None)) if t is not None]
         return ts

@@ -24,6 +24,16 @@ normed input ``h`` and return a sublayer output, with their sizes and constants 
 * :class:`ChunkAttentionMixer` -- softmax attention whose values are the keys as projected; biased q / k
   projections, pairwise rotation with optionally scaled frequencies, weightless per-head RMS norm of q
   and k after the rotation, and a chunked mask (a query sees the keys of its own block of positions).
+* :class:`SigmoidAttentionMixer` -- causal attention without positions and without softmax: independent
+  sigmoid weights sigmoid(score + a bias per head), not normalised over the keys.
+* :class:`MinGRUMixer` -- minimal gated recurrent unit: a diagonal recurrence whose update gate and
+  candidate read only the current token, with a SiLU output gate.
+* :class:`WeightedParallelMixer` -- two mixers side by side whose outputs are summed with fixed weights.
+* :class:`SinkWindowAttentionMixer` -- softmax attention with half-split rotation on part of each head,
+  weightless per-head RMS norm of q and k after the rotation, a sliding window that also keeps the first
+  tokens of the sequence, and values blended with those of the model's first such layer.
+* :class:`PlainLatentAttentionMixer` -- latent attention without positions: keys and values are
+  up-projections of one cached normed latent per token, plain causal softmax.
 * :class:`DenseFF` -- up, activation, down; optionally gated (act(gate) * up).
 * :class:`TopSoftmaxRoutedFF` -- mixture of plain relu^2 experts, softmax over the chosen logits, plus a
   shared expert.
@@ -170,13 +180,13 @@ class LatentAttentionMixer:
 
 
 class DenseFF:
-    """W_down act(W_up h), ``act`` = "relu2" (the square of relu); or, ``gated``,
+    """W_down act(W_up h), ``act`` = "relu2" (the square of relu) | gelu_tanh | silu; or, ``gated``,
     W_down (act(W_gate h) * (W_up h)) with ``act`` in silu | gelu_tanh."""
 
     def __init__(self, spec: Dict, width: int, act: str = "relu2", gated: bool = False):
         self.ff, self.width, self.act, self.gated = int(spec["ff"]), width, act, gated
         self.in_rows = self.ff * (2 if gated else 1)
-        if (act != "relu2") != gated or act not in ("relu2", "silu", "gelu_tanh"):
+        if act not in (("silu", "gelu_tanh") if gated else ("relu2", "silu", "gelu_tanh")):
             raise ValueError(f"unknown activation {act!r} for a {'gated' if gated else 'plain'} feed-forward")
 
     def shapes(self) -> Dict[str, tuple]:
@@ -197,7 +207,8 @@ class DenseFF:
     def forward(self, h: torch.Tensor, proj: torch.Tensor, x32: Optional[torch.Tensor] = None) -> torch.Tensor:
         if self.gated:
             return F.linear(mx.glu_act(proj[:, :self.ff], proj[:, self.ff:2 * self.ff], self.act), self.down)
-        return F.linear(mx.relu2(proj), self.down)
+        up = proj[:, :self.ff]
+        return F.linear(mx.relu2(up) if self.act == "relu2" else mx.glu_act(up, None, self.act), self.down)
 
 
 class RoutedFF:
@@ -778,26 +789,32 @@ class ChunkAttentionMixer:
 class ParallelMixer:
     """Two mixers side by side reading the same input (``left``: windowed attention, ``right``: gated
     LRU block).  ``forward`` returns both outputs; the layer takes half the sum of their RMS norms
-    over the model width, with the plain weights ``left.out`` / ``right.out``."""
+    over the model width, with the plain weights ``left.out`` / ``right.out``.  Subclasses choose other
+    pairs (``left_cls`` / ``right_cls``) and may do without the output norm weights."""
     kind = "parallel"
+    left_cls: type = None        # set below the class definitions
+    right_cls: type = None
+    out_norms = True
 
     def __init__(self, spec: Dict, width: int, eps: float):
-        self.left = WindowAttentionMixer(spec["left"], width, eps)
-        self.right = GatedLRUMixer(spec["right"], width, eps)
+        self.left = self.left_cls(spec["left"], width, eps)
+        self.right = self.right_cls(spec["right"], width, eps)
         self.width = width
         self.in_rows = self.left.in_rows + self.right.in_rows
 
     def shapes(self) -> Dict[str, tuple]:
         s = {f"left.{k}": v for k, v in self.left.shapes().items()}
         s.update({f"right.{k}": v for k, v in self.right.shapes().items()})
-        s.update({"left.out": (self.width,), "right.out": (self.width,)})
+        if self.out_norms:
+            s.update({"left.out": (self.width,), "right.out": (self.width,)})
         return s
 
     def cache_spec(self):
         return ("pair", self.left.cache_spec(), self.right.cache_spec())
 
     def load(self, get: Getter, dtype) -> torch.Tensor:
-        self.out_w = (_f32(get, "left.out"), _f32(get, "right.out"))
+        if self.out_norms:
+            self.out_w = (_f32(get, "left.out"), _f32(get, "right.out"))
         wl = self.left.load(lambda k: get("left." + k), dtype)
         wr = self.right.load(lambda k: get("right." + k), dtype)
         return torch.cat([wl, wr], 0)
@@ -811,7 +828,218 @@ class ParallelMixer:
                 self.right.forward(proj[:, n:], positions, meta, cache[2]))
 
 
+ParallelMixer.left_cls, ParallelMixer.right_cls = WindowAttentionMixer, GatedLRUMixer
+
+
+class SigmoidAttentionMixer:
+    """Causal attention without positions and without softmax.  ``kv_heads`` key/value heads (query head h
+    reads head h // (H/G)), key size ``dim``, value size ``vdim``, no biases on the projections, no
+    rotation; score = q . k * scale; every key j <= i is visible (a ``mask`` entry {size} narrows this to
+    a sliding window) and weighs sigmoid(score + pb[h]) with one bias per query head -- the weights of a
+    query are independent and are not normalised.  W_o on the concatenated heads.  The cache holds one
+    row [k | v] per token."""
+    kind = "sigmoid_attention"
+
+    def __init__(self, spec: Dict, width: int, eps: float):
+        self.H, self.G = int(spec["heads"]), int(spec.get("kv_heads", spec["heads"]))
+        self.D, self.P = int(spec["dim"]), int(spec["vdim"])
+        mask = spec.get("mask") or {}
+        self.window = int(mask["size"]) if mask.get("size") else 1 << 30
+        self.scale = float(spec["scale"]) if "scale" in spec else self.D ** -0.5
+        self.width, self.eps = width, eps
+        if self.H % self.G or self.D > 512 or self.P > 512:
+            raise ValueError("sigmoid attention: heads must split into kv_heads; dim, vdim <= 512")
+        self.nq, self.nk, self.nv = self.H * self.D, self.G * self.D, self.G * self.P
+        self.in_rows = self.nq + self.nk + self.nv
+
+    def shapes(self) -> Dict[str, tuple]:
+        W = self.width
+        return {"q": (self.nq, W), "k": (self.nk, W), "v": (self.nv, W), "pb": (self.H,), "o": (W, self.H * self.P)}
+
+    def cache_spec(self):
+        return ("rows", self.nk + self.nv)
+
+    def load(self, get: Getter, dtype) -> torch.Tensor:
+        self.pb = _f32(get, "pb")
+        self.o = get("o").to(dtype).contiguous()
+        return torch.cat([get("q"), get("k"), get("v")], 0).to(dtype)
+
+    def num_bytes(self) -> int:
+        return self.o.numel() * self.o.element_size()
+
+    def forward(self, proj: torch.Tensor, positions: torch.Tensor, meta: AttentionMetadata, cache) -> torch.Tensor:
+        rows = cache[1]
+        nq, nk, nv = self.nq, self.nk, self.nv
+        q = mx.qk_norm_write(proj[:, :nq], proj[:, nq:nq + nk], proj[:, nq + nk:nq + nk + nv], None, None, self.eps,
+                             meta.slots, rows)
+        o = mx.window_attend(q, rows, meta.seg_cu, positions, meta.seg_bt, self.window, self.scale, meta.seg_max_len,
+                             self.H, self.G, self.D, self.P, head_bias=self.pb)
+        return F.linear(o, self.o)
+
+
+class MinGRUMixer:
+    """Minimal gated recurrent unit of ``width`` channels: z = sigmoid(W_z h + b_z), u = W_x h + b_x, candidate
+    c = u + 1/2 where u >= 0 and sigmoid(u) below; element by element S <- (1 - z) S + z c on an f32 state
+    per sequence that starts at zero (the gates read only the current token); output W_o (S * silu(W_g h))."""
+    kind = "mingru"
+
+    def __init__(self, spec: Dict, width: int, eps: float):
+        self.R = int(spec["width"])
+        self.width, self.eps = width, eps
+        self.in_rows = 3 * self.R
+
+    def shapes(self) -> Dict[str, tuple]:
+        R, W = self.R, self.width
+        return {"z": (R, W), "z.b": (R,), "x": (R, W), "x.b": (R,), "g": (R, W), "o": (W, R)}
+
+    def cache_spec(self):
+        return ("slots", {"S": (self.R,)})
+
+    def load(self, get: Getter, dtype) -> torch.Tensor:
+        self.z_b, self.x_b = _f32(get, "z.b"), _f32(get, "x.b")      # added in f32: they enter the recurrence
+        self.o = get("o").to(dtype).contiguous()
+        return torch.cat([get("z"), get("x"), get("g")], 0).to(dtype)
+
+    def num_bytes(self) -> int:
+        return self.o.numel() * self.o.element_size()
+
+    def forward(self, proj: torch.Tensor, positions: torch.Tensor, meta: AttentionMetadata, cache) -> torch.Tensor:
+        R = self.R
+        s = mx.mingru_scan(proj[:, :R], proj[:, R:2 * R], proj[:, 2 * R:3 * R], self.z_b, self.x_b, cache[1]["S"],
+                           meta.seg_cu, meta.seg_state, positions, proj.dtype, max_len=meta.seg_max_len)
+        return F.linear(s, self.o)
+
+
+class WeightedParallelMixer(ParallelMixer):
+    """Sigmoid attention (``left``) beside a minimal GRU (``right``) on the same input; the layer adds
+    left_scale * left + right_scale * right (``forward`` returns both, ``scales`` the two weights)."""
+    left_cls, right_cls = SigmoidAttentionMixer, MinGRUMixer
+    out_norms = False
+
+    def __init__(self, spec: Dict, width: int, eps: float):
+        super().__init__(spec, width, eps)
+        self.scales = (float(spec.get("left_scale", 1.0)), float(spec.get("right_scale", 1.0)))
+
+
+class SinkWindowAttentionMixer:
+    """Softmax attention with ``kv_heads`` key/value heads (query head h reads head h // (H/G)), no biases.
+    q and k are rotated on the first rot.dims entries of each head (entry i with entry i + dims/2, angle
+    position * base^(-2i/dims), every frequency divided by rot.scaling.factor when given), then each head
+    is divided by its root mean square over dim (no weight); score = q . k * scale; position i sees j <= i
+    with i - j < mask.size or j < mask.keep_first (the kept first tokens stay at their true positions; no
+    ``mask`` entry: plain causal); softmax; W_o.  With ``v_mix`` the values of every such layer but the
+    model's first are blended with the first one's values of the same token,
+    v <- (1 - vmix) v + vmix v_first (``forward``'s ``v_first``), before they are cached.  The cache
+    holds one row [finished k | v] per token."""
+    kind = "sink_window_attention"
+
+    def __init__(self, spec: Dict, width: int, eps: float):
+        self.H, self.G = int(spec["heads"]), int(spec.get("kv_heads", spec["heads"]))
+        self.D, self.P = int(spec["dim"]), int(spec["vdim"])
+        self.rot = _Rotary(spec.get("rot"), self.D)
+        mask = spec.get("mask") or {}
+        self.window = int(mask["size"]) if mask.get("size") else 1 << 30
+        self.keep = int(mask.get("keep_first") or 0) if mask.get("size") else 0
+        self.scale = float(spec["scale"]) if "scale" in spec else self.D ** -0.5
+        self.v_mix = bool(spec.get("v_mix"))
+        self.lam = 0.0
+        self.width, self.eps = width, eps
+        if self.H % self.G or self.D > 512 or self.P > 512:
+            raise ValueError("attention: heads must split into kv_heads; dim, vdim <= 512")
+        self.nq, self.nk, self.nv = self.H * self.D, self.G * self.D, self.G * self.P
+        self.in_rows = self.nq + self.nk + self.nv
+
+    def shapes(self) -> Dict[str, tuple]:
+        W = self.width
+        s = {"q": (self.nq, W), "k": (self.nk, W), "v": (self.nv, W), "o": (W, self.H * self.P)}
+        if self.v_mix:
+            s["vmix"] = ()
+        return s
+
+    def cache_spec(self):
+        return ("rows", self.nk + self.nv)
+
+    def load(self, get: Getter, dtype) -> torch.Tensor:
+        self.o = get("o").to(dtype).contiguous()
+        self.rot.to(self.o.device)
+        if self.v_mix:
+            self.lam = float(get("vmix").float().item())
+        return torch.cat([get("q"), get("k"), get("v")], 0).to(dtype)
+
+    def num_bytes(self) -> int:
+        return self.o.numel() * self.o.element_size()
+
+    def values(self, proj: torch.Tensor) -> torch.Tensor:
+        """This layer's values as projected (what later layers blend theirs with)."""
+        return proj[:, self.nq + self.nk:self.nq + self.nk + self.nv]
+
+    def forward(self, proj: torch.Tensor, positions: torch.Tensor, meta: AttentionMetadata, cache,
+                v_first: Optional[torch.Tensor] = None) -> torch.Tensor:
+        rows = cache[1]
+        nq, nk = self.nq, self.nk
+        q, _ = mx.rope_heads(proj[:, :nq], proj[:, nq:nq + nk], self.H, self.G, self.D, self.rot.freq, positions, "half",
+                             self.rot.mscale, norm_eps=self.eps, k_out=rows, slots=meta.slots, v=self.values(proj),
+                             v_mix=v_first, v_lam=self.lam)
+        o = mx.window_attend(q, rows, meta.seg_cu, positions, meta.seg_bt, self.window, self.scale, meta.seg_max_len,
+                             self.H, self.G, self.D, self.P, keep_first=self.keep)
+        return F.linear(o, self.o)
+
+
+class PlainLatentAttentionMixer:
+    """Latent attention without positions: q = W_q h ([heads, dim]); c = RMSnorm(W_dkv h) * w (``kv_rank``
+    entries, plain weight); per head k = W_uk c, v = W_uv c; score = q . k * scale; plain causal softmax;
+    W_o.  Only c is cached; the kernels run in the latent space (each head's W_uk folded into its query,
+    W_uv applied to the attention output), so all heads read the same cache rows."""
+    kind = "plain_latent_attention"
+
+    def __init__(self, spec: Dict, width: int, eps: float):
+        self.H, self.D, self.P, self.R = int(spec["heads"]), int(spec["dim"]), int(spec["vdim"]), int(spec["kv_rank"])
+        mask = spec.get("mask") or {}
+        self.window = int(mask["size"]) if mask.get("size") else 1 << 30
+        self.scale = float(spec["scale"]) if "scale" in spec else self.D ** -0.5
+        self.width, self.eps = width, eps
+        if self.R > 512:
+            raise ValueError("latent attention: kv_rank <= 512")
+        self.nq = self.H * self.D
+        self.in_rows = self.nq + self.R
+
+    def shapes(self) -> Dict[str, tuple]:
+        W, H = self.width, self.H
+        return {"q": (self.nq, W), "dkv": (self.R, W), "dkv.norm": (self.R,), "uk": (H * self.D, self.R),
+                "uv": (H * self.P, self.R), "o": (W, H * self.P)}
+
+    def cache_spec(self):
+        return ("latent", self.R)
+
+    def load(self, get: Getter, dtype) -> torch.Tensor:
+        self.dkv_norm = _f32(get, "dkv.norm")
+        self.uk = get("uk").to(dtype).view(self.H, self.D, self.R).contiguous()                       # [H, D, R]
+        self.uv_t = get("uv").to(dtype).view(self.H, self.P, self.R).transpose(1, 2).contiguous()     # [H, R, P]
+        self.o = get("o").to(dtype).contiguous()
+        self.no_freq = torch.zeros(0, dtype=torch.float32, device=self.o.device)
+        return torch.cat([get("q"), get("dkv")], 0).to(dtype)
+
+    def num_bytes(self) -> int:
+        return sum(t.numel() * t.element_size() for t in (self.uk, self.uv_t, self.o))
+
+    def forward(self, proj: torch.Tensor, positions: torch.Tensor, meta: AttentionMetadata, cache) -> torch.Tensor:
+        rows = cache[1]
+        T = proj.shape[0]
+        H, D, R = self.H, self.D, self.R
+        q = proj[:, :self.nq]
+        # the normed latent into the cache (no rotated part: the returned rotated query part is empty)
+        q_rot = mx.latent_prep(proj[:, self.nq:self.nq + R], self.dkv_norm, self.eps, self.no_freq, 0, positions,
+                               meta.slots, rows, q, H, D, D, R, 0)
+        q_lat = torch.bmm(q.reshape(T, H, D).transpose(0, 1), self.uk).transpose(0, 1).contiguous()     # [T, H, R]
+        o_lat = mx.latent_attend(q_lat, q_rot, rows, meta.seg_cu, positions, meta.seg_bt, self.window, self.scale,
+                                 meta.seg_max_len)
+        o = torch.bmm(o_lat.transpose(0, 1), self.uv_t).transpose(0, 1).reshape(T, H * self.P)
+        return F.linear(o, self.o)
+
+
 MIXERS = {"mamba2": Mamba2Mixer, "latent_attention": LatentAttentionMixer, "channel_delta": ChannelDeltaMixer,
           "gla": GLAMixer, "window_attention": WindowAttentionMixer, "gated_lru": GatedLRUMixer,
           "parallel": ParallelMixer, "lightning": LightningMixer, "retention": RetentionMixer,
-          "attention": ChunkAttentionMixer}
+          "attention": ChunkAttentionMixer, "sigmoid_attention": SigmoidAttentionMixer, "mingru": MinGRUMixer,
+          "weighted_parallel": WeightedParallelMixer, "sink_window_attention": SinkWindowAttentionMixer,
+          "plain_latent_attention": PlainLatentAttentionMixer}

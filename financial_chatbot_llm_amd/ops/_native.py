@@ -86,7 +86,8 @@ c_double = ctypes.c_double
 # its own -- a model that runs only these builds and loads only these
 _MIXER_SIGS = {
     "mx_embed": [P, P, c_int, P, c_int, c_int, c_int, P],
-    "mx_residual_norm": [P, P, c_long, P, c_long, c_int, c_float, P, c_float, P, c_int, c_int, c_int, P],
+    "mx_residual_norm": [P, P, c_long, P, c_long, c_int, c_float, c_float, P, c_long, P, P, c_float, P, c_int, c_int,
+                         c_int, P],
     "mx_group_norm": [P, c_long, c_int, P, c_long, c_int, P, c_float, P, c_long, c_int, c_int, c_int, c_int, P],
     "mx_relu2": [P, c_long, P, c_long, c_int, c_int, c_int, P],
     "mx_glu_clamp": [P, c_long, P, c_long, c_float, c_float, P, c_long, c_int, c_int, c_int, P],
@@ -103,14 +104,16 @@ _MIXER_SIGS = {
                        P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P],
     "mx_lru_scan": [P, P, c_int, P, P, P, P, c_long, c_int, P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P],
     "mx_qk_norm_write": [P, c_long, P, c_long, P, c_long, P, P, c_float, P, P, P, c_int, c_int, c_int, c_int, c_int, P],
-    "mx_window_attend": [P, c_long, P, P, P, P, c_int, P, c_long, c_int, c_int, c_float, P, c_int, c_int, c_int, c_int,
-                         c_int, c_int, c_int, c_int, P, P],
+    "mx_window_attend": [P, c_long, P, P, P, P, c_int, P, c_long, c_int, c_int, c_int, P, c_float, P, c_int, c_int, c_int,
+                         c_int, c_int, c_int, c_int, c_int, P, P],
+    "mx_mingru_scan": [P, c_long, P, c_long, P, c_long, c_int, P, P, P, P, P, P, P, P, P, c_int, c_int, c_int, c_int,
+                       c_int, P],
     "mx_decay_scan": [P, c_long, P, c_long, c_int, P, c_long, c_int, c_int, P, c_float, P, P, P, P, P, c_int, c_int,
                       c_int, c_int, c_int, c_int, P],
     "mx_embed_scaled": [P, P, c_int, c_float, c_int, P, c_int, c_int, c_int, P],
     "mx_hyper_mix": [P, P, c_long, c_int, P, P, P, P, c_float, P, c_int, c_int, c_int, c_int, P],
     "mx_rope_heads": [P, c_long, c_int, P, c_long, c_int, c_int, c_int, c_int, c_int, P, c_float, P, c_int, c_float,
-                      c_float, c_float, P, c_int, P, c_long, c_int, P, P, c_long, c_int, c_int, P],
+                      c_float, c_float, P, c_int, P, c_long, c_int, P, P, c_long, c_int, P, c_long, c_float, c_int, P],
     "mx_logit_cap": [P, c_int, c_float, c_float, c_long, P],
     "mx_ssm_scan": [P, c_int, P, c_long, c_int, P, P, P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, P],
     "mx_latent_prep": [P, c_long, P, c_float, P, c_int, P, P, P, P, c_long, c_int, c_int, P, c_int, c_int, c_int,

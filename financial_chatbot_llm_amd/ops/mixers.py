@@ -63,27 +63,38 @@ def embed_f32(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
 
 def residual_norm(x: torch.Tensor, w: Optional[torch.Tensor], eps: float, a: Optional[torch.Tensor] = None,
                   b: Optional[torch.Tensor] = None, mult: float = 1.0,
-                  out_dtype: torch.dtype = torch.bfloat16) -> Optional[torch.Tensor]:
+                  out_dtype: torch.dtype = torch.bfloat16, mult_b: Optional[float] = None,
+                  gate: Optional[torch.Tensor] = None, gate_bias: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
     """``x`` (f32 [T, W], in place) <- x + mult * (a + b) when a sublayer output is given, then
-    y = x / sqrt(mean(x^2) + eps) * w in ``out_dtype`` (``w`` None: the update only)."""
+    y = x / sqrt(mean(x^2) + eps) * w in ``out_dtype`` (``w`` None: the update only).  ``mult_b``: b's own
+    weight, the update is mult * a + mult_b * b.  ``gate`` ([T, W] column slice, the type of a) and
+    ``gate_bias`` (f32 [W]): the update is multiplied element by element by sigmoid(gate + gate_bias)."""
     T, W = x.shape
     assert x.dtype == torch.float32 and x.is_contiguous()
     ab = a if a is not None else b
+    mult_b = mult if mult_b is None else mult_b
+    if gate is not None and ab is None:
+        raise ValueError("a gate needs a sublayer output to act on")
     if N.use_native(x):
         out = torch.empty((T, W), dtype=out_dtype, device=x.device) if w is not None else None
         if a is not None and b is not None:
             assert a.dtype == b.dtype
+        if gate is not None:
+            assert gate.dtype == ab.dtype and gate.shape[1] == W
         N.mcall("mx_residual_norm", N.ptr(x), N.ptr(_rows(a)) if a is not None else None,
                 a.stride(0) if a is not None else 0, N.ptr(_rows(b)) if b is not None else None,
-                b.stride(0) if b is not None else 0, _dt(ab) if ab is not None else 1, float(mult),
-                N.ptr(w), float(eps), N.ptr(out), _dt(out) if out is not None else 1, T, W, N.stream())
+                b.stride(0) if b is not None else 0, _dt(ab) if ab is not None else 1, float(mult), float(mult_b),
+                N.ptr(_rows(gate)) if gate is not None else None, gate.stride(0) if gate is not None else 0,
+                N.ptr(gate_bias), N.ptr(w), float(eps), N.ptr(out), _dt(out) if out is not None else 1, T, W, N.stream())
         return out
     if ab is not None:
         s = torch.zeros_like(x)
-        for t in (a, b):
+        for t, m in ((a, mult), (b, mult_b)):
             if t is not None:
-                s = s + t.float()
-        x.add_(mult * s)
+                s = s + m * t.float()
+        if gate is not None:
+            s = s * torch.sigmoid(gate.float() + (gate_bias.float() if gate_bias is not None else 0.0))
+        x.add_(s)
     if w is None:
         return None
     return (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w.float()).to(out_dtype)
@@ -447,18 +458,24 @@ def _act(v: torch.Tensor, act: str) -> torch.Tensor:
     return v
 
 
-def glu_act(gate: torch.Tensor, up: torch.Tensor, act: str, row_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+def glu_act(gate: torch.Tensor, up: Optional[torch.Tensor], act: str,
+            row_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
     """act(s * gate) * (s * up) with ``s`` an optional f32 scale per row (a routed expert whose weight
-    multiplies its INPUT: the scale commutes with the two projections); ``act``: silu | gelu_tanh."""
+    multiplies its INPUT: the scale commutes with the two projections); ``act``: silu | gelu_tanh | sigmoid.
+    ``up`` None: act(s * gate) alone (a plain, ungated feed-forward)."""
     T, n = gate.shape
     if N.use_native(gate):
         out = torch.empty((T, n), dtype=gate.dtype, device=gate.device)
-        N.mcall("mx_glu_act", N.ptr(_rows(gate)), gate.stride(0), N.ptr(_rows(up)), up.stride(0), N.ptr(row_scale),
-                ACTS[act], N.ptr(out), out.stride(0), _dt(gate), T, n, N.stream())
+        N.mcall("mx_glu_act", N.ptr(_rows(gate)), gate.stride(0), N.ptr(_rows(up)) if up is not None else None,
+                up.stride(0) if up is not None else 0, N.ptr(row_scale), ACTS[act], N.ptr(out), out.stride(0), _dt(gate),
+                T, n, N.stream())
         return out
-    g, u = gate.float(), up.float()
+    g = gate.float()
     if row_scale is not None:
-        g, u = g * row_scale[:, None], u * row_scale[:, None]
+        g = g * row_scale[:, None]
+    if up is None:
+        return _act(g, act).to(gate.dtype)
+    u = up.float() * (row_scale[:, None] if row_scale is not None else 1.0)
     return (_act(g, act) * u).to(gate.dtype)
 
 
@@ -654,6 +671,46 @@ def lru_scan(u: torch.Tensor, z: torch.Tensor, blocks: int, r_bias: torch.Tensor
 
 
 # ----------------------------------------------------------------------------------------------
+# minimal gated recurrent unit
+# ----------------------------------------------------------------------------------------------
+def mingru_scan(zp: torch.Tensor, xp: torch.Tensor, gp: torch.Tensor, z_bias: Optional[torch.Tensor],
+                x_bias: Optional[torch.Tensor], state: torch.Tensor, cu: torch.Tensor, slot: torch.Tensor,
+                pos: torch.Tensor, out_dtype: torch.dtype, max_len: int = 0) -> torch.Tensor:
+    """Per channel, f32: z = sigmoid(zp + z_bias), u = xp + x_bias, candidate c = u + 1/2 where u >= 0 and
+    sigmoid(u) below, S <- (1 - z) S + z c (gates from the current token only); returns S * silu(gp) in
+    ``out_dtype``.  ``zp``, ``xp``, ``gp`` [T, R] are column slices of one projection; ``state`` f32
+    [slots, R], read unless the segment starts at position 0, then replaced.  ``max_len``: the longest
+    segment when known (1 selects the fused single-row kernel)."""
+    T, R = zp.shape
+    S = cu.numel() - 1
+    assert xp.shape == zp.shape == gp.shape and zp.dtype == xp.dtype == gp.dtype
+    if N.use_native(zp):
+        out = torch.empty((T, R), dtype=out_dtype, device=zp.device)
+        one = max_len == 1
+        ab = None if one else torch.empty((T, 2 * R), dtype=torch.float32, device=zp.device)
+        gy = None if one else torch.empty((T, R), dtype=torch.float32, device=zp.device)
+        N.mcall("mx_mingru_scan", N.ptr(_rows(zp)), zp.stride(0), N.ptr(_rows(xp)), xp.stride(0), N.ptr(_rows(gp)),
+                gp.stride(0), _dt(zp), N.ptr(z_bias), N.ptr(x_bias), N.ptr(ab), N.ptr(gy), N.ptr(state), N.ptr(cu),
+                N.ptr(slot), N.ptr(pos), N.ptr(out), _dt(out), S, R, T, int(max_len), N.stream())
+        return out
+    a = zp.float() + (z_bias.float() if z_bias is not None else 0.0)
+    u = xp.float() + (x_bias.float() if x_bias is not None else 0.0)
+    keep, put = torch.sigmoid(-a), torch.sigmoid(a) * torch.where(u >= 0, u + 0.5, torch.sigmoid(u))
+    out = torch.zeros((T, R), dtype=torch.float32)
+    cul, sll, pl = cu.tolist(), slot.tolist(), pos.tolist()
+    for s in range(S):
+        r0, r1 = cul[s], cul[s + 1]
+        if sll[s] < 0 or r1 <= r0:
+            continue
+        St = torch.zeros(R) if pl[r0] == 0 else state[sll[s]].clone()
+        for t in range(r0, r1):
+            St = keep[t] * St + put[t]
+            out[t] = St
+        state[sll[s]] = St
+    return (out * F.silu(gp.float())).to(out_dtype)
+
+
+# ----------------------------------------------------------------------------------------------
 # sliding-window attention with grouped key/value heads over a paged row cache
 # ----------------------------------------------------------------------------------------------
 def qk_norm_write(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, qw: Optional[torch.Tensor],
@@ -680,17 +737,22 @@ def qk_norm_write(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, qw: Optiona
 
 def window_attend(q: torch.Tensor, cache: torch.Tensor, cu: torch.Tensor, pos: torch.Tensor, bt: torch.Tensor,
                   window: int, scale: float, max_len: int, heads: int, kv_heads: int, dim: int, vdim: int,
-                  gate: Optional[torch.Tensor] = None, chunked: bool = False) -> torch.Tensor:
+                  gate: Optional[torch.Tensor] = None, chunked: bool = False, keep_first: int = 0,
+                  head_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Causal softmax attention of ``q`` [T, H*dim] over the cache rows [k: G*dim | v: G*vdim] of each
     segment's pages: the query at position p sees keys j with 0 <= p - j < window, or -- ``chunked`` --
     the keys j <= p with floor(j / window) == floor(p / window) (blocks of ``window`` positions counted
-    from the start of the sequence); query head h
-    reads key/value head h // (H/G); score = q . k * scale, f32 softmax; head h's output is
-    multiplied by sigmoid(gate[t, h]) when a gate [T, H] is given.  Returns [T, H*vdim]."""
+    from the start of the sequence); with ``keep_first`` the keys j < keep_first of the sequence stay
+    visible to every later query as well (at their true positions).  Query head h
+    reads key/value head h // (H/G); score = q . k * scale, f32 softmax -- or, with ``head_bias`` (f32 [H]),
+    no softmax: the weight of a visible key is sigmoid(score + head_bias[h]), not normalised over the keys.
+    Head h's output is multiplied by sigmoid(gate[t, h]) when a gate [T, H] is given.  Returns [T, H*vdim]."""
     T = q.shape[0]
     H, G, D, P = heads, kv_heads, dim, vdim
     S = cu.numel() - 1
     Wr = G * (D + P)
+    if head_bias is not None and (head_bias.dtype != torch.float32 or head_bias.numel() != H):
+        raise ValueError("head_bias: one f32 value per query head")
     if N.use_native(q):
         assert bt.is_contiguous() and q.dtype == cache.dtype
         out = torch.empty((T, H * P), dtype=q.dtype, device=q.device)
@@ -698,14 +760,14 @@ def window_attend(q: torch.Tensor, cache: torch.Tensor, cu: torch.Tensor, pos: t
         # small batch still fills the chip; the split depends only on static sizes (graph-safe)
         nsplit, ws = 1, None
         if max_len == 1 and q.dtype == torch.bfloat16:
-            tiles = (min(window, bt.shape[1] * PAGE) + 31) // 32 + 1
+            tiles = (min(window + keep_first, bt.shape[1] * PAGE) + 31) // 32 + 1
             nsplit = max(1, min(16, tiles // 2, 1024 // max(S * G, 1)))
             if nsplit > 1:
                 ws = torch.empty((T, H, nsplit, P + 2), dtype=torch.float32, device=q.device)
         N.mcall("mx_window_attend", N.ptr(_rows(q)), q.stride(0), N.ptr(cache), N.ptr(cu), N.ptr(pos), N.ptr(bt), bt.shape[1],
                 N.ptr(_rows(gate)) if gate is not None else None, gate.stride(0) if gate is not None else 0,
-                int(min(window, 1 << 30)), 1 if chunked else 0, float(scale), N.ptr(out), _dt(q), S, int(max_len), H, G,
-                D, P, nsplit, N.ptr(ws), N.stream())
+                int(min(window, 1 << 30)), 1 if chunked else 0, int(keep_first), N.ptr(head_bias), float(scale), N.ptr(out),
+                _dt(q), S, int(max_len), H, G, D, P, nsplit, N.ptr(ws), N.stream())
         return out
     out = torch.zeros((T, H, P), dtype=torch.float32)
     rows = cache.view(-1, Wr).float()
@@ -723,9 +785,12 @@ def window_attend(q: torch.Tensor, cache: torch.Tensor, cu: torch.Tensor, pos: t
         sc = torch.einsum("nhd,jhd->nhj", q[a:b].float().view(-1, H, D), keys) * scale
         p = pos[a:b].long()[:, None]
         j = torch.arange(ctx)[None]
-        vis = (j <= p) & ((j // window == p // window) if chunked else (j > p - window))
-        sc = sc.masked_fill(~vis[:, None, :], float("-inf"))
-        out[a:b] = torch.einsum("nhj,jhp->nhp", torch.softmax(sc, -1), vals)
+        vis = (j <= p) & (((j // window == p // window) if chunked else (j > p - window)) | (j < keep_first))
+        if head_bias is not None:
+            wt = torch.sigmoid(sc + head_bias.float()[None, :, None]) * vis[:, None, :]
+        else:
+            wt = torch.softmax(sc.masked_fill(~vis[:, None, :], float("-inf")), -1)
+        out[a:b] = torch.einsum("nhj,jhp->nhp", wt, vals)
     if gate is not None:
         out = out * torch.sigmoid(gate.float())[:, :, None]
     return out.reshape(T, H * P).to(q.dtype)
@@ -799,12 +864,15 @@ def rope_freqs(dims: int, base: float, scaling: Optional[dict] = None, device=No
     ``scaling`` entry {factor, original, fast, slow} (YaRN): with turn(t) = dims ln(original / (2 pi t)) /
     (2 ln base), lo = max(floor(turn(fast)), 0), hi = min(ceil(turn(slow)), dims - 1) and
     ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1) the frequency is f_i / factor * ramp_i +
-    f_i (1 - ramp_i) and cos and sin are multiplied by 0.1 ln(factor) + 1."""
+    f_i (1 - ramp_i) and cos and sin are multiplied by 0.1 ln(factor) + 1.  A ``scaling`` entry with a factor
+    only is linear scaling: every f_i is divided by the factor (positions are stretched), cos and sin unscaled."""
     import math
     i = torch.arange(dims // 2, dtype=torch.float64)
     f = float(base) ** (-2.0 * i / dims)
     m = 1.0
-    if scaling:
+    if scaling and "original" not in scaling:      # linear scaling: every frequency divided by the factor
+        f = f / float(scaling["factor"])
+    elif scaling:
         factor, orig = float(scaling["factor"]), float(scaling["original"])
         turn = lambda t: dims * math.log(orig / (2 * math.pi * float(t))) / (2 * math.log(float(base)))  # noqa: E731
         lo = max(math.floor(turn(scaling["fast"])), 0)
@@ -836,7 +904,8 @@ def rope_heads(q: torch.Tensor, k: torch.Tensor, heads: int, kv_heads: int, dim:
                pos: torch.Tensor, layout: str = "pairs", mscale: float = 1.0, norm_eps: Optional[float] = None,
                q_scale: float = 1.0, k_scale: float = 1.0, q_dtype: Optional[torch.dtype] = None,
                k_out: Optional[torch.Tensor] = None, slots: Optional[torch.Tensor] = None,
-               v: Optional[torch.Tensor] = None, k_dtype: Optional[torch.dtype] = None):
+               v: Optional[torch.Tensor] = None, k_dtype: Optional[torch.dtype] = None,
+               v_mix: Optional[torch.Tensor] = None, v_lam: float = 0.0):
     """Per head of ``q`` [T, H*dim] and ``k`` [T, G*dim] (column slices): the first ``2 * len(freq)``
     entries are rotated by the angle pos * freq_i (f32), pair i being entries (2i, 2i+1) for
     ``layout="pairs"`` or (i, i + rot/2) for ``"half"``; (u, v) -> (u cos - v sin, v cos + u sin) with cos and
@@ -844,7 +913,8 @@ def rope_heads(q: torch.Tensor, k: torch.Tensor, heads: int, kv_heads: int, dim:
     ``dim`` (no weight); then times ``q_scale`` / ``k_scale``.  Returns (q', k'): q' [T, H*dim] in
     ``q_dtype``; k' [T, G*dim] in ``k_dtype`` -- or, with ``k_out`` (paged cache rows [rows, G*dim + nv])
     and ``slots`` [T], k' is written to row slots[t] (< 0: no write) followed by the raw values ``v``
-    [T, nv], and None is returned for it."""
+    [T, nv], and None is returned for it; with ``v_mix`` ([T, nv]) the values written are
+    (1 - v_lam) v + v_lam v_mix, blended in f32."""
     T = q.shape[0]
     H, G, D = heads, kv_heads, dim
     rot = 2 * freq.numel() if freq is not None else 0
@@ -862,11 +932,14 @@ def rope_heads(q: torch.Tensor, k: torch.Tensor, heads: int, kv_heads: int, dim:
         else:
             nv = v.shape[1] if v is not None else 0
             assert k_out.shape[-1] >= G * D + nv and k_out.stride(-1) == 1 and slots is not None
+            assert v_mix is None or (v is not None and v_mix.shape == v.shape and v_mix.dtype == v.dtype)
             ko, dst, sko, sl = None, k_out, k_out.shape[-1], slots
         N.mcall("mx_rope_heads", N.ptr(_rows(q)), q.stride(0), H, N.ptr(_rows(k)), k.stride(0), G, _dt(q), D, rot,
                 1 if half else 0, N.ptr(freq), float(mscale), N.ptr(pos), 1 if norm else 0, float(norm_eps or 0.0),
                 float(q_scale), float(k_scale), N.ptr(qo), _dt(qo), N.ptr(dst), sko, _dt(dst), N.ptr(sl),
-                N.ptr(_rows(v)) if v is not None else None, v.stride(0) if v is not None else 0, nv, T, N.stream())
+                N.ptr(_rows(v)) if v is not None else None, v.stride(0) if v is not None else 0, nv,
+                N.ptr(_rows(v_mix)) if v_mix is not None else None, v_mix.stride(0) if v_mix is not None else 0,
+                float(v_lam), T, N.stream())
         return qo, ko
     ang = pos.float()[:, None] * freq.float()[None, :] if rot else None
 
@@ -880,7 +953,10 @@ def rope_heads(q: torch.Tensor, k: torch.Tensor, heads: int, kv_heads: int, dim:
     kk = prep(k, G, k_scale)
     if k_out is None:
         return qo, kk.to(k_dtype or k.dtype)
-    rows = torch.cat([kk] + ([v.float()] if v is not None else []), 1).to(k_out.dtype)
+    vv = v.float() if v is not None else None
+    if v_mix is not None:
+        vv = (1.0 - v_lam) * vv + v_lam * v_mix.float()
+    rows = torch.cat([kk] + ([vv] if vv is not None else []), 1).to(k_out.dtype)
     ok = slots >= 0
     k_out.view(-1, k_out.shape[-1])[slots[ok].long(), :rows.shape[1]] = rows[ok]
     return qo, None
