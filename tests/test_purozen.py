@@ -1,0 +1,654 @@
+"""Purozen (pre-norm layered decoder with sigmoid-gated residual updates and a tied vocabulary projection)
+against the plain oracle of tests/purozen_oracle.py.
+
+Small configurations with random weights made here; the framework side always runs through the engine
+(scheduler admission, pages, state slots, runner) or the ops' public entry points.  CPU tensors exercise
+the ops' PyTorch forms, ``cuda`` ones the HIP kernels (marked gpu).
+"""
+import copy
+
+import numpy as np
+import pytest
+import torch
+
+import purozen_oracle as oracle
+from financial_chatbot_llm_amd.config import EngineConfig
+from financial_chatbot_llm_amd.engine import LLMEngine, SamplingParams
+from financial_chatbot_llm_amd.models.configs import layered_config
+from financial_chatbot_llm_amd.models.purozen import PurozenModel, example_config
+from financial_chatbot_llm_amd.ops import mixers as mx
+
+DEVICES = ["cpu", pytest.param("cuda", marks=pytest.mark.gpu)]
+DTYPES = [torch.float32, torch.bfloat16]
+TOL = {torch.float32: 3e-4, torch.bfloat16: 8e-2}
+
+
+def random_weights(model, seed):
+    g = torch.Generator().manual_seed(seed)
+    sd = {}
+    for name, shape in model.full_shapes().items():
+        leaf = name.rsplit(".", 1)[-1]
+        r = torch.randn(shape, generator=g)
+        if leaf in ("norm1", "norm2") or name == "final.norm":
+            t = 0.2 * r                                  # stored around zero
+        elif leaf == "norm":
+            t = 1.0 + 0.2 * r
+        elif leaf == "vmix":
+            t = torch.rand((), generator=g) * 0.6 + 0.2
+        elif leaf == "pb":
+            t = r - 1.0
+        elif leaf == "b" and len(shape) == 1:
+            t = 0.5 * r
+        elif leaf == "embed":
+            t = r
+        else:
+            t = r * shape[-1] ** -0.5 * 1.3
+        sd[name] = t.to(torch.bfloat16)
+    return sd
+
+
+def small_config(pattern="paAl", **over):
+    return example_config(width=over.pop("width", 96), vocab=over.pop("vocab", 160), pattern=pattern)
+
+
+def build(cfgd, device, dtype, seed=1, blocks_=24, seqs=4, graphs=False, async_=False, max_len=1024):
+    mc = layered_config(cfgd, "purozen-test")
+    model = PurozenModel(mc, device=device, dtype=dtype)
+    sd = random_weights(model, seed)
+    model.load_state(sd)
+    eng = LLMEngine(EngineConfig(model="purozen-test", device=device, dtype="fp32" if dtype == torch.float32 else "bf16",
+                                 num_kv_blocks=blocks_, max_num_seqs=seqs, max_model_len=max_len,
+                                 max_num_batched_tokens=512, enable_prefix_caching=False, use_cuda_graph=graphs,
+                                 async_scheduling=async_, graph_batch_sizes=(1, 2, 4)), model=model)
+    return eng, sd
+
+
+def _poison(entry):
+    for t in entry[1:]:
+        if isinstance(t, dict):
+            for v in t.values():
+                v.fill_(float("nan"))
+        elif isinstance(t, tuple):
+            _poison(t)
+        else:
+            t.fill_(float("nan"))
+
+
+def poison(eng):
+    """Pages and slots as a previous owner might have left them: nothing may depend on their content."""
+    for lay in eng.kv.layers:
+        _poison(lay)
+
+
+def close(got, want, dtype):
+    got, want = torch.as_tensor(got).double().cpu(), torch.as_tensor(want).double()
+    assert torch.isfinite(got).all()
+    err = (got - want).abs().flatten(1).max(-1).values / max(want.abs().max().item(), 1e-9)
+    assert err.max() <= TOL[dtype], f"{int((err > TOL[dtype]).sum())} of {err.numel()} positions over: worst {err.max():.3e}"
+
+
+def tokens(n, vocab, seed):
+    return torch.randint(0, vocab, (n,), generator=torch.Generator().manual_seed(seed)).tolist()
+
+
+def run_whole(eng, rid, toks):
+    return eng.replay_step([(rid, toks, list(range(len(toks))))], [rid])
+
+
+def i32(x, device="cpu"):
+    return torch.tensor(x, dtype=torch.int32, device=device)
+
+
+# ---------------------------------------------------------------------------------------------------
+# each mechanism alone: one-layer models
+# ---------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("pattern", ["p", "a", "l", "P", "aa"])
+def test_one_mechanism_against_oracle(device, dtype, pattern):
+    """One layer per kind ("aa": the second layer blends its values with the first one's)."""
+    cfgd = small_config(pattern)
+    eng, sd = build(cfgd, device, dtype)
+    poison(eng)
+    toks = tokens(90, cfgd["vocab"], 3)          # crosses a 64-token page and leaves the 37-token window twice
+    close(run_whole(eng, "r", toks), oracle.forward(cfgd, sd, toks), dtype)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_residual_stream_after_every_layer(device):
+    cfgd = small_config("paAl")
+    eng, sd = build(cfgd, device, torch.float32)
+    toks = tokens(40, cfgd["vocab"], 4)
+    want = []
+    oracle.forward(cfgd, sd, toks, want)
+    eng.model.capture = []
+    run_whole(eng, "r", toks)
+    assert len(eng.model.capture) == len(want) == 4
+    for got, ref in zip(eng.model.capture, want):
+        close(got, ref, torch.float32)
+
+
+def test_mechanism_functions_alone():
+    """The ops' reference forms against the oracle's functions on raw projections (no engine): the two
+    branches of the recurrent unit's candidate, the gated residual update with two weighted outputs."""
+    g = torch.Generator().manual_seed(0)
+    T, R = 30, 10
+    zp, xp, gp = (2.0 * torch.randn(T, R, generator=g) for _ in range(3))
+    zb, xb = torch.randn(R, generator=g), torch.randn(R, generator=g)
+    state = torch.full((2, R), float("nan"))
+    out = mx.mingru_scan(zp, xp, gp, zb, xb, state, i32([0, T]), i32([1]), torch.arange(T, dtype=torch.int32), torch.float32, T)
+    eye = np.eye(R)
+    w = {"z": eye, "x": eye, "g": eye, "o": eye, "z.b": zb.double().numpy(), "x.b": xb.double().numpy()}
+    # the oracle reads h through W_z, W_x, W_g: feed each projection on its own through identity weights
+    z = oracle.sigmoid(zp.double().numpy() + w["z.b"])
+    u = xp.double().numpy() + w["x.b"]
+    assert (u >= 0).any() and (u < 0).any()
+    cand = np.where(u >= 0, u + 0.5, oracle.sigmoid(u))
+    S, want = np.zeros(R), np.zeros((T, R))
+    for t in range(T):
+        S = (1 - z[t]) * S + z[t] * cand[t]
+        want[t] = S * gp[t].double().numpy() * oracle.sigmoid(gp[t].double().numpy())
+    assert np.abs(out.double().numpy() - want).max() < 1e-5
+    assert np.abs(state[1].double().numpy() - S).max() < 1e-5 and torch.isnan(state[0]).all()
+    # gated update: x + sigmoid(gate + bias) * (0.7 a + 1.2 b), then the norm with its finished weight
+    x = torch.randn(T, R, generator=g)
+    a, b, gate = (torch.randn(T, R, generator=g) for _ in range(3))
+    bias, wn = torch.randn(R, generator=g), torch.randn(R, generator=g)
+    x0 = x.clone()
+    h = mx.residual_norm(x, 1.0 + wn, 1e-3, a=a, b=b, mult=0.7, mult_b=1.2, gate=gate, gate_bias=bias, out_dtype=torch.float32)
+    xw = x0.double().numpy() + oracle.sigmoid((gate + bias).double().numpy()) * (0.7 * a.double().numpy() + 1.2 * b.double().numpy())
+    assert np.abs(x.double().numpy() - xw).max() < 1e-5
+    assert np.abs(h.double().numpy() - oracle.norm(xw, wn.double().numpy(), 1e-3)).max() < 1e-5
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_absent_entries_and_single_sizes(device):
+    """No feed-forward, no mask, no rotation, no frequency scaling, no value blending, a single blending
+    layer, one head, one key/value head, as many key/value heads as heads, keep_first 0 and 1, a window of
+    one key, scales of 0 and 1."""
+    cfgd = small_config("aAapPal")
+    L = cfgd["layers"]
+    del L[0]["mixer"]["mask"]
+    del L[0]["mixer"]["rot"]["scaling"]
+    L[0]["mixer"].update(heads=1, kv_heads=1, v_mix=False)
+    del L[1]["mixer"]["rot"]
+    L[1]["mixer"]["mask"] = {"size": 1, "keep_first": 0}
+    L[1]["mixer"].update(kv_heads=6)
+    del L[1]["mixer"]["v_mix"]
+    L[2]["mixer"]["mask"] = {"size": 5, "keep_first": 1}          # the only blending layer: nothing to blend with
+    L[3]["mixer"]["left"].update(heads=1, kv_heads=1)
+    L[3]["mixer"].update(left_scale=1.0, right_scale=0.0)
+    L[4]["mixer"]["left"].update(kv_heads=6)
+    L[4]["mixer"].update(left_scale=0.0, right_scale=1.0)
+    L[5]["mixer"]["mask"] = {"size": 9}                           # no keep_first entry
+    L[5]["mixer"].update(v_mix=False)
+    L[6]["mixer"].update(heads=1)
+    eng, sd = build(cfgd, device, torch.float32)
+    assert "l1.norm2" not in sd and "l1.rg2" not in sd and "l0.mix.vmix" not in sd and "l2.mix.vmix" in sd
+    poison(eng)
+    toks = tokens(70, cfgd["vocab"], 5)
+    close(run_whole(eng, "r", toks), oracle.forward(cfgd, sd, toks), torch.float32)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_other_sizes(device, dtype):
+    """Sizes unlike the small default: odd head counts, key and value sizes that fill no wave and differ,
+    a window longer than a page and one shorter than the kept first tokens, rotation over the whole head
+    and over two entries, the first blending layer behind an attention layer that does not blend, three
+    blending layers, a large norm eps, other constants."""
+    cfgd = small_config("alapaPaL", width=80, vocab=97)
+    cfgd["norm"]["eps"] = 0.02
+    L = cfgd["layers"]
+    L[0]["mixer"].update(dim=40, vdim=9, heads=6, kv_heads=1, mask={"size": 70, "keep_first": 2}, scale=0.31, v_mix=False,
+                         rot={"base": 777.0, "dims": 40})
+    L[1]["mixer"].update(dim=9, vdim=33, heads=3, kv_rank=50, scale=0.6)
+    L[2]["mixer"].update(dim=18, vdim=10, heads=4, kv_heads=4, mask={"size": 3, "keep_first": 7}, scale=2.0,
+                         rot={"base": 50.0, "dims": 2, "scaling": {"factor": 1.5}})
+    L[3]["mixer"]["left"].update(dim=12, vdim=34, heads=5, kv_heads=5, scale=0.4)
+    L[3]["mixer"]["right"].update(width=50)
+    L[3]["mixer"].update(left_scale=1.3, right_scale=0.4)
+    L[4]["mixer"].update(dim=34, vdim=20, heads=2, kv_heads=2, mask={"size": 100, "keep_first": 100}, scale=0.8,
+                         rot={"base": 1e6, "dims": 34, "scaling": {"factor": 8.0}})
+    L[5]["mixer"]["left"].update(dim=132, vdim=17, heads=2, kv_heads=1, scale=0.05)
+    L[5]["mixer"]["right"].update(width=3)
+    L[6]["mixer"].update(dim=16, vdim=8, heads=5, kv_heads=5, mask={"size": 64, "keep_first": 64}, scale=1.0)
+    L[7]["mixer"].update(dim=70, vdim=5, heads=2, kv_rank=9, scale=0.2)
+    eng, sd = build(cfgd, device, dtype, blocks_=8)
+    poison(eng)
+    toks = tokens(150, cfgd["vocab"], 7)
+    close(run_whole(eng, "r", toks), oracle.forward(cfgd, sd, toks), dtype)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_wide_heads(device, dtype):
+    """Head and latent sizes beyond what the matrix-core kernels cover (bf16 then takes the f32-lane kernels)."""
+    cfgd = small_config("apl", width=64)
+    L = cfgd["layers"]
+    L[0]["mixer"].update(dim=264, vdim=264, heads=2, kv_heads=1, scale=0.9, rot={"base": 1000.0, "dims": 200})
+    L[1]["mixer"]["left"].update(dim=260, vdim=40, heads=2, kv_heads=2, scale=0.05)
+    L[2]["mixer"].update(kv_rank=330, heads=2)
+    eng, sd = build(cfgd, device, dtype, blocks_=4)
+    toks = tokens(80, cfgd["vocab"], 8)
+    close(run_whole(eng, "r", toks), oracle.forward(cfgd, sd, toks), dtype)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_first_tokens(device):
+    """Sequences of one and two tokens, and the first tokens of a longer one, each request alone."""
+    cfgd = small_config("paal")
+    eng, sd = build(cfgd, device, torch.float32)
+    poison(eng)
+    for n in (1, 2, 5):
+        toks = tokens(n, cfgd["vocab"], 60 + n)
+        close(run_whole(eng, f"r{n}", toks), oracle.forward(cfgd, sd, toks), torch.float32)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("pattern", ["aAl", "pP"])
+def test_single_mixer_kind_models(device, pattern):
+    """Only attention layers (no state slots at all) and only parallel layers."""
+    cfgd = small_config(pattern)
+    eng, sd = build(cfgd, device, torch.float32)
+    poison(eng)
+    assert (eng.state_slots is None) == (pattern == "aAl")
+    toks = tokens(100, cfgd["vocab"], 17)
+    want = oracle.forward(cfgd, sd, toks)
+    got = [eng.replay_step([("r", toks[:70], list(range(70)))])]
+    got += [eng.replay_step([("r", toks[i:i + 1], [0])]) for i in range(70, 100)]
+    close(torch.cat(got), want, torch.float32)
+
+
+# ---------------------------------------------------------------------------------------------------
+# cache, state, batching
+# ---------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_prefill_then_token_by_token(device, dtype):
+    cfgd = small_config("paal")
+    eng, sd = build(cfgd, device, dtype)
+    poison(eng)
+    toks = tokens(140, cfgd["vocab"], 11)
+    want = oracle.forward(cfgd, sd, toks)
+    got = [eng.replay_step([("r", toks[:30], list(range(30)))])]
+    for i in range(30, len(toks)):               # long decoding: the window passes over decoded tokens and a page border
+        got.append(eng.replay_step([("r", toks[i:i + 1], [0])], ["r"] if i == len(toks) - 1 else []))
+    close(torch.cat(got), want, dtype)
+    assert eng.bm.num_free() == eng.bm.num_blocks and eng.state_slots.num_free() == 4
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("sizes", [[2, 2, 3, 60, 2, 1, 1, 64, 5], [63, 1, 1, 2, 70], [1, 1, 1, 130], [2] * 20, [36, 2, 36, 1, 37]])
+def test_portions(device, sizes):
+    """Portions cut inside pages and inside windows, down to two tokens."""
+    cfgd = small_config("apal")
+    eng, sd = build(cfgd, device, torch.float32)
+    poison(eng)
+    toks = tokens(sum(sizes), cfgd["vocab"], 13)
+    want = oracle.forward(cfgd, sd, toks)
+    got, at = [], 0
+    for n in sizes:
+        got.append(eng.replay_step([("r", toks[at:at + n], list(range(n)))]))
+        at += n
+    close(torch.cat(got), want, torch.float32)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_mixed_batches_and_reuse(device, dtype):
+    """Unequal requests in one batch (portions beside single tokens), more requests than slots and a
+    pool that only fits what is live: pages and slots are freed and used again."""
+    cfgd = small_config("apla")
+    eng, sd = build(cfgd, device, dtype, blocks_=7, seqs=3)
+    poison(eng)
+    V = cfgd["vocab"]
+    reqs = {f"q{i}": tokens(n, V, 20 + i) for i, n in enumerate([150, 70, 33, 100, 5, 64])}
+    want = {k: torch.as_tensor(oracle.forward(cfgd, sd, t)) for k, t in reqs.items()}
+    got = {k: [] for k in reqs}
+    at = {k: 0 for k in reqs}
+    sched = [
+        [("q0", 50), ("q1", 3), ("q2", 33)],            # q2 complete at once
+        [("q0", 1), ("q1", 60), ("q3", 2)],             # q3 takes q2's slot and pages
+        [("q0", 30), ("q1", 1), ("q3", 62)],
+        [("q1", 1), ("q0", 69), ("q3", 1)],
+        [("q1", 5), ("q3", 35)],                        # q1, q3, q0 complete
+        [("q4", 5), ("q5", 2)],
+        [("q5", 62)],
+    ]
+    for step in sched:
+        entries, end = [], []
+        for k, n in step:
+            entries.append((k, reqs[k][at[k]:at[k] + n], list(range(n))))
+            at[k] += n
+            if at[k] == len(reqs[k]):
+                end.append(k)
+        out = eng.replay_step(entries, end)
+        o = 0
+        for k, t, _ in entries:
+            got[k].append(out[o:o + len(t)])
+            o += len(t)
+    assert eng.state_slots.reuses > 0
+    assert all(at[k] == len(reqs[k]) for k in reqs)
+    close(torch.cat([torch.cat(got[k]) for k in reqs]), torch.cat([want[k] for k in reqs]), dtype)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_batch_rows_do_not_depend_on_their_neighbours(device):
+    """The same request alone and between two others gives the same logits (f32)."""
+    cfgd = small_config("pal")
+    eng, sd = build(cfgd, device, torch.float32)
+    V = cfgd["vocab"]
+    a, b, c = tokens(45, V, 1), tokens(20, V, 2), tokens(70, V, 3)
+    alone = run_whole(eng, "x", b)
+    poison(eng)
+    out = eng.replay_step([("a", a, []), ("b", b, list(range(len(b)))), ("c", c, [])], ["a", "b", "c"])
+    assert (out - alone).abs().max() <= 2e-6 * alone.abs().max()
+
+
+# ---------------------------------------------------------------------------------------------------
+# window edges, kept first tokens, page borders, far keys: scores and states that stand out
+# ---------------------------------------------------------------------------------------------------
+def _paged(n, pages, width, g, table):
+    row = lambda j: int(table[0, j // 64]) * 64 + j % 64  # noqa: E731
+    cache = torch.zeros(pages * 64, width)
+    return cache, row
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("size,keep", [(5, 2), (64, 3), (70, 20), (33, 64), (40, 0)])
+def test_window_and_kept_edges_stand_out(device, dtype, size, keep):
+    """One key per query gets an overwhelming score and the output must be that key's value exactly when
+    the key is visible: the oldest key of the window (seen) and the one before it (not seen, unless
+    kept), the last kept key (seen from anywhere) and the first key that is not kept (seen only through
+    the window).  Queries are rows of a prompt chunk and single decoded rows, around page borders;
+    three query heads share each of two key/value heads."""
+    H, G, D, P, pages, n = 6, 2, 16, 12, 4, 200
+    g = torch.Generator().manual_seed(size)
+    table = i32([[2, 0, 3, 1]])
+    cache, row = _paged(n, pages, G * (D + P), g, table)
+    for j in range(n):
+        cache[row(j), G * D:] = torch.randn(G * P, generator=g)           # values; keys stay zero
+    chunks = [list(range(p0, p0 + 8)) for p0 in (size + keep, 60, 124, 188)]
+    chunks += [[p] for p in (size - 1, size, size + keep, 63, 64, 65, 127, 128, 199)]
+    kinds = ["oldest", "before", "first_not_kept"] + (["last_kept"] if keep else [])
+    for kind in kinds:
+        for seg in chunks:
+            m = len(seg)
+            kc = cache.clone()
+            q = torch.zeros(m, H, D)
+            target = []
+            for i, p in enumerate(seg):          # query i asks for key coordinate i; only its target key is large there
+                t = {"oldest": max(p - size + 1, 0), "before": p - size, "last_kept": min(keep - 1, p),
+                     "first_not_kept": min(keep, p)}[kind]
+                target.append(t)
+                if t >= 0:
+                    for kvh in range(G):
+                        kc[row(t), kvh * D + i] = 50.0
+                q[i, :, i] = 4.0
+            out = mx.window_attend(q.reshape(m, H * D).to(dtype).to(device), kc.to(dtype).to(device), i32([0, m], device),
+                                   i32(seg, device), table.to(device), size, 1.0, m, H, G, D, P,
+                                   keep_first=keep).float().cpu().view(m, H, P)
+            kcr = kc.to(dtype).float()
+            for i, p in enumerate(seg):
+                vis = [j for j in range(p + 1) if p - j < size or j < keep]
+                rows_ = [row(j) for j in vis]
+                for h in range(H):
+                    kvh = h // (H // G)
+                    pr = torch.softmax(kcr[rows_, kvh * D + i] * 4.0, 0)
+                    ref = (pr[:, None] * kcr[rows_, G * D + kvh * P:G * D + (kvh + 1) * P]).sum(0)
+                    tol = 1e-4 if dtype == torch.float32 else 0.05
+                    assert (out[i, h] - ref).abs().max() < tol, (kind, seg, i, h)
+                    if target[i] >= 0:
+                        tv = kcr[row(target[i]), G * D + kvh * P:G * D + (kvh + 1) * P]
+                        assert bool((out[i, h] - tv).abs().max() < 0.05) == (target[i] in vis), (kind, seg, i, h)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_far_keys_softmax_and_sigmoid(device):
+    """One far key among hundreds carries the score, seen from a chunk deep in the sequence and from
+    single rows (also where a single row's keys are split over several blocks): under plain causal
+    softmax, as a kept first token behind a short window, and under sigmoid weights, where it adds to
+    the near keys instead of replacing them; a short window without kept tokens hides it."""
+    H, G, D, P = 4, 2, 24, 8
+    n, pages, far = 400, 8, 7
+    g = torch.Generator().manual_seed(2)
+    perm = torch.randperm(pages, generator=g).to(torch.int32)[None]
+    rows = 0.1 * torch.randn(n, G * (D + P), generator=g)
+    rows[far, 1] = rows[far, D + 1] = 30.0                 # both key heads, coordinate 1
+    rows[far, G * D:] = 9.0
+    cache = torch.zeros(pages * 64, G * (D + P))
+    for j in range(n):
+        cache[int(perm[0, j // 64]) * 64 + j % 64] = rows[j]
+    pos = torch.arange(330, 400, dtype=torch.int32)
+    q = torch.zeros(len(pos), H, D)
+    q[:, :, 1] = 3.0
+    cu = i32([0, len(pos)])
+    for size, keep, hit in ((1 << 30, 0, True), (16, 8, True), (16, 7, False), (320, 0, False), (393, 0, True)):
+        out = mx.window_attend(q.view(len(pos), -1).to(device), cache.to(device), cu.to(device), pos.to(device),
+                               perm.to(device), size, 1.0, len(pos), H, G, D, P, keep_first=keep).cpu()
+        assert bool((out > 8.0).all()) == hit and bool((out < 8.0).all()) == (not hit)
+        for dt in DTYPES:
+            one = mx.window_attend(q[:1].view(1, -1).to(dt).to(device), cache.to(dt).to(device), i32([0, 1], device),
+                                   i32([399], device), perm.to(device), size, 1.0, 1, H, G, D, P,
+                                   keep_first=keep).float().cpu()
+            assert bool((one > 8.0).all()) == hit
+    # a window the far key leaves in the middle of the chunk: rows at positions < 7 + 340 still see it
+    out = mx.window_attend(q.view(len(pos), -1).to(device), cache.to(device), cu.to(device), pos.to(device),
+                           perm.to(device), 340, 1.0, len(pos), H, G, D, P).cpu()
+    assert bool((out[:17] > 8.0).all()) and bool((out[17:] < 8.0).all())
+    # sigmoid weights: the bias silences the ordinary keys (score ~ 0 -> sigmoid(-12)), the far key passes
+    bias = torch.full((H,), -12.0)
+    for dt in DTYPES:
+        c = cache.to(dt).to(device)
+        out = mx.window_attend(q.view(len(pos), -1).to(dt).to(device), c, cu.to(device), pos.to(device), perm.to(device),
+                               1 << 30, 1.0, len(pos), H, G, D, P, head_bias=bias.to(device)).float().cpu()
+        one = mx.window_attend(q[:1].view(1, -1).to(dt).to(device), c, i32([0, 1], device), i32([399], device),
+                               perm.to(device), 1 << 30, 1.0, 1, H, G, D, P, head_bias=bias.to(device)).float().cpu()
+        for o in (out, one):
+            assert (o - 9.0).abs().max() < 0.1             # weight 1 on the far key, ~6e-6 on each of the others
+    # weights are not normalised: with a large bias every visible key weighs one and the output is the plain sum
+    big = torch.full((H,), 30.0)
+    out = mx.window_attend(q[:3].view(3, -1).to(device), cache.to(device), i32([0, 3], device), i32([9, 10, 11], device),
+                           perm.to(device), 1 << 30, 1.0, 3, H, G, D, P, head_bias=big.to(device)).cpu().view(3, H, P)
+    for i, p in enumerate((9, 10, 11)):
+        want = rows[:p + 1, G * D:].view(p + 1, G, P).sum(0)
+        assert (out[i, 0] - want[0]).abs().max() < 1e-3 and (out[i, H - 1] - want[G - 1]).abs().max() < 1e-3
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_sigmoid_weights_against_plain_sums(device, dtype):
+    """Sigmoid attention rows of a chunk and decoded rows against a direct evaluation, one bias per head,
+    more than one page, grouped heads."""
+    H, G, D, P, n = 6, 3, 20, 9, 150
+    g = torch.Generator().manual_seed(5)
+    table = i32([[1, 2, 0]])
+    rows = torch.randn(n, G * (D + P), generator=g).to(dtype)
+    cache = torch.zeros(3 * 64, G * (D + P), dtype=dtype)
+    for j in range(n):
+        cache[int(table[0, j // 64]) * 64 + j % 64] = rows[j]
+    bias = torch.randn(H, generator=g) - 2.0
+    for seg in (list(range(100, 150)), [149], [64], [0]):
+        m = len(seg)
+        q = torch.randn(m, H, D, generator=g).to(dtype)
+        out = mx.window_attend(q.view(m, -1).to(device), cache.to(device), i32([0, m], device), i32(seg, device),
+                               table.to(device), 1 << 30, 0.3, m, H, G, D, P, head_bias=bias.to(device)).float().cpu().view(m, H, P)
+        for i, p in enumerate(seg):
+            k = rows[:p + 1, :G * D].float().view(p + 1, G, D).repeat_interleave(H // G, 1)
+            v = rows[:p + 1, G * D:].float().view(p + 1, G, P).repeat_interleave(H // G, 1)
+            wt = torch.sigmoid(torch.einsum("hd,jhd->hj", q[i].float(), k) * 0.3 + bias[:, None])
+            ref = torch.einsum("hj,jhp->hp", wt, v)
+            assert (out[i] - ref).abs().max() < (1e-4 if dtype == torch.float32 else 0.08) * max(ref.abs().max().item(), 1.0)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_recurrent_state_keeps_a_far_write(device):
+    """A candidate written 300 tokens back under update gates that stay shut is still the state at the end,
+    through portions that hand the state over in a reused slot; a channel whose gates are open forgets it."""
+    R, n = 6, 300
+    big = 30.0
+    zp = torch.full((n, R), -big)
+    zp[5] = big                                   # token 5 writes every channel
+    zp[6:, 3:] = 0.0                              # channels 3.. keep updating (z = 1/2): they forget
+    xp = torch.zeros(n, R)
+    xp[5] = 2.0                                   # candidate 2.5
+    gp = torch.full((n, R), big)                  # silu(30) = 30
+    state = torch.full((3, R), float("nan"))
+    st = state.to(device)
+    outs, at = [], 0
+    for m in (4, 2, 60, 1, 1, 130, 2, 100):       # the write sits in a two-token portion
+        seg = slice(at, at + m)
+        outs.append(mx.mingru_scan(zp[seg].to(device), xp[seg].to(device), gp[seg].to(device), None, None, st,
+                                   i32([0, m], device), i32([2], device),
+                                   torch.arange(at, at + m, dtype=torch.int32, device=device), torch.float32, m).cpu())
+        at += m
+    out = torch.cat(outs)
+    assert (out[:5].abs() < 1e-6).all()                               # from zero, whatever the slot held
+    assert (out[5:, :3] / big - 2.5).abs().max() < 1e-3               # kept over 294 tokens
+    assert (out[-1, 3:] / big - 0.5).abs().max() < 1e-3               # forgotten: the state of candidate 1/2
+    assert torch.isnan(st[:2]).all().item()                           # other slots untouched
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_segments_around_the_scan_kernel_sizes(device):
+    """Several segments per step with lengths on and around the recurrence kernel's chunk sizes, starting
+    states from slots, against a token-by-token evaluation."""
+    R = 37
+    g = torch.Generator().manual_seed(9)
+    lens = [1, 15, 16, 17, 255, 256, 257, 600, 2]
+    T = sum(lens)
+    zp, xp, gp = (torch.randn(T, R, generator=g) for _ in range(3))
+    zb, xb = torch.randn(R, generator=g), torch.randn(R, generator=g)
+    start = torch.randn(len(lens), R, generator=g)
+    cu = [0]
+    for n_ in lens:
+        cu.append(cu[-1] + n_)
+    pos = torch.cat([torch.arange(n_) + (0 if s % 3 == 0 else 11) for s, n_ in enumerate(lens)]).to(torch.int32)
+    st = start.clone().to(device)
+    out = mx.mingru_scan(zp.to(device), xp.to(device), gp.to(device), zb.to(device), xb.to(device), st, i32(cu, device),
+                         i32(list(range(len(lens))), device), pos.to(device), torch.float32, max(lens)).cpu()
+    z = torch.sigmoid(zp.double() + zb.double())
+    u = xp.double() + xb.double()
+    cand = torch.where(u >= 0, u + 0.5, torch.sigmoid(u))
+    for s, n_ in enumerate(lens):
+        S = torch.zeros(R, dtype=torch.float64) if s % 3 == 0 else start[s].double()
+        for t in range(cu[s], cu[s + 1]):
+            S = (1 - z[t]) * S + z[t] * cand[t]
+            assert (out[t].double() - S * gp[t].double() * torch.sigmoid(gp[t].double())).abs().max() < 2e-5, (s, t)
+        assert (st[s].cpu().double() - S).abs().max() < 2e-5
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rotation_scaling_and_value_blend(device, dtype):
+    """Half-split rotation on part of the head with linearly scaled frequencies at large positions, the
+    weightless norm after it, and the blended values in the cache row."""
+    H, G, D, P, T, rot, eps = 3, 1, 20, 7, 9, 12, 1e-3
+    g = torch.Generator().manual_seed(3)
+    freq, m = mx.rope_freqs(rot, 500.0, {"factor": 4.0})
+    assert m == 1.0 and torch.allclose(freq.double(), 500.0 ** (-2.0 * torch.arange(rot // 2).double() / rot) / 4.0, rtol=1e-6)
+    q, k = torch.randn(T, H * D, generator=g).to(dtype), torch.randn(T, G * D, generator=g).to(dtype)
+    v, v1 = torch.randn(T, G * P, generator=g).to(dtype), torch.randn(T, G * P, generator=g).to(dtype)
+    pos = torch.tensor([0, 1, 2, 63, 64, 1000, 2049, 3000, 4097], dtype=torch.int32)   # angles are f32: up to ~1e3 rad
+    slots = i32([3, -1, 0, 1, 2, 7, 6, 5, 4])
+    rows = torch.zeros(8, G * (D + P), dtype=dtype)
+    rows_d = rows.to(device)
+    qo, _ = mx.rope_heads(q.to(device), k.to(device), H, G, D, freq.to(device), pos.to(device), "half", 1.0, norm_eps=eps,
+                          k_out=rows_d, slots=slots.to(device), v=v.to(device), v_mix=v1.to(device), v_lam=0.3)
+    rd = {"base": 500.0, "dims": rot, "scaling": {"factor": 4.0}}
+
+    def want(x, nh):
+        out = np.zeros((T, nh, D))
+        x = x.double().numpy().reshape(T, nh, D)
+        for t in range(T):           # the oracle rotates by the row index: evaluate each position on its own
+            pad = np.zeros((int(pos[t]) + 1, nh, D))
+            pad[-1] = x[t]
+            out[t] = oracle.rms(oracle.rotate_half(pad, rd), eps)[-1]
+        return out.reshape(T, nh * D)
+
+    tol = 3e-4 if dtype == torch.float32 else 3e-2
+    assert np.abs(qo.float().cpu().numpy() - want(q, H)).max() < tol
+    kw, vw = want(k, G), 0.7 * v.double().numpy() + 0.3 * v1.double().numpy()
+    got = rows_d.float().cpu().numpy()
+    for t in range(T):
+        if slots[t] >= 0:
+            assert np.abs(got[slots[t], :G * D] - kw[t]).max() < tol and np.abs(got[slots[t], G * D:] - vw[t]).max() < tol
+
+
+# ---------------------------------------------------------------------------------------------------
+# generation through the engine's own scheduler
+# ---------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("device,graphs", [("cpu", False), pytest.param("cuda", False, marks=pytest.mark.gpu),
+                                           pytest.param("cuda", True, marks=pytest.mark.gpu)])
+@pytest.mark.parametrize("async_", [False, True])
+def test_greedy_generation(device, graphs, async_):
+    cfgd = small_config("paal", vocab=256)
+    eng, sd = build(cfgd, device, torch.float32, blocks_=12, seqs=2, graphs=graphs, async_=async_)
+    poison(eng)
+    prompts = [tokens(70, 256, 41), tokens(9, 256, 42), tokens(30, 256, 43)]     # three requests, two slots
+    outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True))
+    for p, o in zip(prompts, outs):
+        assert o == oracle.greedy(cfgd, sd, p, 12)
+    assert eng.state_slots.num_free() == 2 and eng.bm.num_free() == eng.bm.num_blocks
+    if graphs:
+        assert eng.runner.stats["graph_steps"] > 0
+
+
+@pytest.mark.gpu
+def test_sampling_from_the_tied_projection():
+    """A width the fused LM-head sampler accepts: it reads the embedding table as the vocabulary projection."""
+    cfgd = small_config("pa", width=256, vocab=512)
+    eng, sd = build(cfgd, "cuda", torch.bfloat16)
+    assert eng.model.lm_weight() is eng.model.embed
+    prompt = tokens(20, 512, 1)
+    outs = eng.generate([prompt], SamplingParams(temperature=0.0, max_tokens=4, ignore_eos=True))
+    assert len(outs[0]) == 4
+
+
+def test_preemption_recomputes_state():
+    """A pool too small for both sequences: the younger one is preempted, gives its slot back and is
+    recomputed from its first token."""
+    cfgd = small_config("pa", vocab=256)
+    eng, sd = build(cfgd, "cpu", torch.float32, blocks_=3, seqs=2)
+    prompts = [tokens(60, 256, 51), tokens(62, 256, 52)]
+    outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True))
+    assert eng.scheduler.num_preemptions > 0
+    for p, o in zip(prompts, outs):
+        assert o == oracle.greedy(cfgd, sd, p, 10)
+
+
+def test_registry_and_config_errors():
+    from financial_chatbot_llm_amd.models import get_model_config
+    c = get_model_config("purozen-tiny")
+    assert c.arch == "purozen" and len(c.layers) == c.num_layers
+    bad = copy.deepcopy(example_config())
+    bad["layers"][0]["type"] = "gla"                 # a mixer of another design
+    with pytest.raises(ValueError):
+        PurozenModel(layered_config(bad, "bad"), device="cpu")
+    bad = copy.deepcopy(example_config())
+    bad["layers"][0]["mlp"]["kind"] = "other"
+    with pytest.raises(ValueError):
+        PurozenModel(layered_config(bad, "bad"), device="cpu")
+    bad = copy.deepcopy(example_config(pattern="aa"))
+    bad["layers"][1]["mixer"]["vdim"] = 20           # blended values must have one size
+    with pytest.raises(ValueError):
+        PurozenModel(layered_config(bad, "bad"), device="cpu")
+    bad = copy.deepcopy(example_config())
+    bad["layers"][1]["mixer"]["heads"] = 5           # heads must split into kv_heads
+    with pytest.raises(ValueError):
+        PurozenModel(layered_config(bad, "bad"), device="cpu")
+    m = PurozenModel(layered_config(example_config(), "ok"), device="cpu")
+    sd = random_weights(m, 0)
+    assert "head" not in sd and "l0.rg1.b" in sd and "l2.rg2" not in sd
+    m.load_state(sd)
+    short = dict(sd)
+    short["l0.rg1"] = sd["l0.rg1"][:1]
+    with pytest.raises(ValueError):
+        m.load_state(short)
+    short = dict(sd)
+    short.pop("l0.mix.left.pb")
+    with pytest.raises(KeyError):
+        m.load_state(short)
+    m.init_random(seed=3)                            # registry examples run with random weights
