@@ -87,10 +87,10 @@ def parse(argv=None):
                          "the step's all-reduce volume priced at stated xGMI rates -- a projection, never a "
                          "multi-GPU measurement")
     ap.add_argument("--json-out", default="")
-    ap.add_argument("--model-throughput", default="", metavar="DESIGN", choices=["", "gezavik", "sigudra", "tukedra"],
+    ap.add_argument("--model-throughput", default="", metavar="DESIGN", choices=["", "gezavik", "sigudra", "tukedra", "purozen"],
                     help="instead of the serving workload: prefill and decode tokens/s of the named layered design at "
                          "a few layer sizes beside its closest relative of equal size (gezavik: a Llama twin; sigudra: "
-                         "Gezavik; tukedra: Sigudra) (bench/model_throughput.py; one JSON "
+                         "Gezavik; tukedra: Sigudra; purozen: a Sigudra with dense feed-forwards) (bench/model_throughput.py; one JSON "
                          "line per model and workload)")
     from financial_chatbot_llm_amd.bench.model_throughput import add_arguments
     add_arguments(ap)

@@ -1,6 +1,6 @@
 """Times the sequence-mixer kernels (``ops.mixers``) at the layer shapes of a hybrid decoder.
 
-    python -m financial_chatbot_llm_amd.bench.mixer_kernels [--width 2048] [--design gezavik|sigudra|tukedra]
+    python -m financial_chatbot_llm_amd.bench.mixer_kernels [--width 2048] [--design gezavik|sigudra|tukedra|purozen]
 
 Two step shapes: a prefill step of two 2048-token prompts and a decode step of 64 single rows at
 depth 1024.  Shapes follow ``models.gezavik.example_config(scale_up=True)``: Mamba-2 with inner =
@@ -13,6 +13,10 @@ gated linear attention, a gated LRU as wide as the model, window 1024).  ``--des
 design's kernels at ``models.tukedra.example_config(scale_up=True)`` shapes (width / 128 heads; lightning
 128 x 128 with the SiLU at staging, retention 64 x 128 on rotated f32 q and k, chunk-masked attention with
 128-wide heads, 4 query heads per key/value head and blocks of 2048 positions; two residual streams).
+``--design purozen``: that design's kernels at ``models.purozen.example_config(scale_up=True)`` shapes
+(width / 128 heads of 128 with 4 query heads per key/value head: sigmoid-weight attention over the whole
+prefix, softmax attention with 64 rotated entries, window 1024 and 4 kept first tokens; a minimal GRU as
+wide as the model; position-free latent attention of rank 256; the gated residual update; plain GeLU).
 """
 from __future__ import annotations
 
@@ -181,11 +185,89 @@ def tukedra(width: int) -> int:
     return 0
 
 
+def purozen(width: int) -> int:
+    dev = "cuda"
+    H, D, P, window, keep, R = max(width // 128, 2), 128, 128, 1024, 4, 256
+    G = max(H // 4, 1)
+    out = lambda **kw: print(json.dumps(kw), flush=True)  # noqa: E731
+    for name, lens, start, cu, pos, slot in _steps(dev):
+        S, T, ml = len(lens), sum(lens), max(lens)
+        pages = (start + ml + 63) // 64
+        bt = torch.arange(S * pages, dtype=torch.int32, device=dev).view(S, pages).contiguous()
+        slots = (bt[:, None, :].expand(S, ml, pages).reshape(-1, pages).gather(1, (pos // 64).long()[:, None])[:, 0] * 64
+                 + pos % 64).to(torch.int32)
+        # sigmoid attention: cache write, then weights sigmoid(score + bias) over the whole prefix
+        cache = torch.randn(S * pages * 64, G * (D + P), device=dev).bfloat16()
+        qkv = torch.randn(T, (H + 2 * G) * D, device=dev).bfloat16() * .1
+        q, k, v = qkv[:, :H * D], qkv[:, H * D:(H + G) * D], qkv[:, (H + G) * D:]
+        us = _time(lambda: mx.qk_norm_write(q, k, v, None, None, 1e-5, slots, cache))
+        out(shape=name, kernel="qk_norm_write (cache write only)", us=round(us, 1),
+            TB_per_s=round(T * 2 * G * (D + P) * 2 / us / 1e6, 2))
+        qc = mx.qk_norm_write(q, k, v, None, None, 1e-5, slots, cache)
+        pb = torch.full((H,), -4.0, device=dev)
+        us = _time(lambda: mx.window_attend(qc, cache, cu, pos, bt, 1 << 30, D ** -0.5, ml, H, G, D, P, head_bias=pb), 5)
+        pairs = sum(p + 1 for n in lens for p in range(start, start + n))
+        out(shape=name, kernel="window_attend sigmoid, causal", us=round(us, 1),
+            bf16_TFLOP_per_s=round(pairs * H * 2 * (D + P) / us / 1e6, 1),
+            cache_TB_per_s=round(S * (start + ml) * G * (D + P) * 2 / us / 1e6, 3))
+        us = _time(lambda: mx.window_attend(qc, cache, cu, pos, bt, 1 << 30, D ** -0.5, ml, H, G, D, P), 5)
+        out(shape=name, kernel="window_attend softmax, causal (same walk)", us=round(us, 1),
+            bf16_TFLOP_per_s=round(pairs * H * 2 * (D + P) / us / 1e6, 1),
+            cache_TB_per_s=round(S * (start + ml) * G * (D + P) * 2 / us / 1e6, 3))
+        # minimal GRU as wide as the model
+        zxg = torch.randn(T, 3 * width, device=dev).bfloat16()
+        zb = torch.zeros(width, device=dev)
+        st = torch.zeros(S, width, device=dev)
+        us = _time(lambda: mx.mingru_scan(zxg[:, :width], zxg[:, width:2 * width], zxg[:, 2 * width:], zb, zb, st, cu, slot, pos,
+                                          torch.bfloat16, max_len=ml))
+        out(shape=name, kernel="mingru_scan", us=round(us, 1), TB_per_s=round(T * width * (8 + 24 + 2) / us / 1e6, 2))
+        # attention: rotation + per-head norm + blended values + cache write, then window + kept first tokens
+        freq, ms = mx.rope_freqs(64, 10000.0, {"factor": 2.0}, device=dev)
+        v1 = torch.randn(T, G * P, device=dev).bfloat16()
+        us = _time(lambda: mx.rope_heads(q, k, H, G, D, freq, pos, "half", ms, norm_eps=1e-5, k_out=cache, slots=slots, v=v,
+                                         v_mix=v1, v_lam=0.3))
+        out(shape=name, kernel="rope_heads + value blend", us=round(us, 1),
+            TB_per_s=round(T * (2 * H * D + 2 * G * D + 3 * G * P) * 2 / us / 1e6, 2))
+        qn, _ = mx.rope_heads(q, k, H, G, D, freq, pos, "half", ms, norm_eps=1e-5, k_out=cache, slots=slots, v=v, v_mix=v1,
+                              v_lam=0.3)
+        us = _time(lambda: mx.window_attend(qn, cache, cu, pos, bt, window, 1.0, ml, H, G, D, P, keep_first=keep), 5)
+        pairs = sum(min(p + 1, window) + (keep if p >= window + keep else 0) for n in lens for p in range(start, start + n))
+        out(shape=name, kernel="window_attend window + kept", us=round(us, 1),
+            bf16_TFLOP_per_s=round(pairs * H * 2 * (D + P) / us / 1e6, 1),
+            cache_TB_per_s=round(S * min(start + ml, window + ml + keep) * G * (D + P) * 2 / us / 1e6, 3))
+        # latent attention without positions, plain causal
+        lcache = torch.randn(S * pages * 64, R, device=dev).bfloat16()
+        kvp = torch.randn(T, R, device=dev).bfloat16()
+        nw = torch.ones(R, device=dev)
+        nof = torch.zeros(0, device=dev)
+        us = _time(lambda: mx.latent_prep(kvp, nw, 1e-5, nof, 0, pos, slots, lcache, q, H, D, D, R, 0))
+        out(shape=name, kernel="latent_prep (no rotation)", us=round(us, 1), TB_per_s=round(T * R * 4 / us / 1e6, 2))
+        ql = torch.randn(T, H, R, device=dev).bfloat16() * .1
+        qr = torch.empty(T, H, 0, device=dev, dtype=torch.bfloat16)
+        us = _time(lambda: mx.latent_attend(ql, qr, lcache, cu, pos, bt, 1 << 30, 0.1, ml), 5)
+        pairs = sum(p + 1 for n in lens for p in range(start, start + n))
+        out(shape=name, kernel="latent_attend causal", us=round(us, 1),
+            bf16_TFLOP_per_s=round(pairs * H * 2 * 2 * R / us / 1e6, 1),
+            cache_TB_per_s=round(S * (start + ml) * R * 2 / us / 1e6, 3))
+        # gated residual update + next norm; plain GeLU on a column slice
+        x = torch.randn(T, width, device=dev)
+        ag = torch.randn(T, 2 * width, device=dev).bfloat16()
+        w = torch.ones(width, device=dev)
+        us = _time(lambda: mx.residual_norm(x, w, 1e-5, a=ag[:, :width], gate=ag[:, width:], gate_bias=zb))
+        out(shape=name, kernel="residual_norm gated", us=round(us, 1), TB_per_s=round(T * width * 14 / us / 1e6, 2))
+        up = torch.randn(T, 5 * width, device=dev).bfloat16()
+        us = _time(lambda: mx.glu_act(up[:, :4 * width], None, "gelu_tanh"))
+        out(shape=name, kernel="gelu_tanh", us=round(us, 1), TB_per_s=round(T * 4 * width * 4 / us / 1e6, 2))
+    return 0
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--width", type=int, default=2048)
-    ap.add_argument("--design", default="gezavik", choices=["gezavik", "sigudra", "tukedra"])
+    ap.add_argument("--design", default="gezavik", choices=["gezavik", "sigudra", "tukedra", "purozen"])
     a = ap.parse_args(argv)
+    if a.design == "purozen":
+        return purozen(a.width)
     if a.design == "sigudra":
         return sigudra(a.width)
     if a.design == "tukedra":

@@ -3,6 +3,7 @@
     python bench.py --model-throughput gezavik [--mt-widths 1024,2048,4096]
     python bench.py --model-throughput sigudra          # beside Gezavik, its closest relative here
     python bench.py --model-throughput tukedra          # beside Sigudra, its closest relative here
+    python bench.py --model-throughput purozen          # beside a dense-feed-forward Sigudra of equal size
     python -m financial_chatbot_llm_amd.bench.model_throughput --mt-only gezavik-w2048
 
 For each width a Gezavik model (random weights, 8 layers: latent attention and Mamba-2 mixers, dense
@@ -96,6 +97,21 @@ def register_tukedra(width: int, vocab: int = 32768) -> List[str]:
     return [name, register_sigudra(width, vocab)[0]]
 
 
+def register_purozen(width: int, vocab: int = 32768) -> List[str]:
+    """Register ``purozen-w<width>`` (8 layers ``paalpaal``: sigmoid attention beside a minimal GRU, windowed
+    attention with kept first tokens and blended values, position-free latent attention; plain GeLU
+    feed-forwards of 4 x width; gated residual updates) and ``sigudra-dense-w<width>``, the Sigudra model of
+    the same width, depth and vocabulary with dense feed-forwards only (``pgpdpgpd``: windowed attention
+    beside a gated LRU, matrix-state scans; within 3 % of the same parameter count); returns the two names."""
+    from ..models.configs import REGISTRY, layered_config
+    from ..models.purozen import example_config
+    from ..models.sigudra import example_config as sigudra_config
+    name, twin = f"purozen-w{width}", f"sigudra-dense-w{width}"
+    REGISTRY[name] = layered_config(example_config(width=width, vocab=vocab, pattern="paalpaal", scale_up=True), name)
+    REGISTRY[twin] = layered_config(sigudra_config(width=width, vocab=vocab, pattern="pgpdpgpd", scale_up=True), twin)
+    return [name, twin]
+
+
 def _tokens(n: int, vocab: int, seed: int) -> List[int]:
     g = torch.Generator().manual_seed(seed)
     return torch.randint(5, vocab - 300, (n,), generator=g).tolist()
@@ -167,7 +183,7 @@ def run(a) -> int:
     names: List[str] = []
     design = getattr(a, "model_throughput", "") or "gezavik"
     for w in (int(x) for x in a.mt_widths.split(",") if x):
-        names += {"sigudra": register_sigudra, "tukedra": register_tukedra}.get(design, register)(w)
+        names += {"sigudra": register_sigudra, "tukedra": register_tukedra, "purozen": register_purozen}.get(design, register)(w)
     if a.mt_only:
         names = [n for n in names if n == a.mt_only]
     for n in names:
@@ -178,7 +194,7 @@ def run(a) -> int:
 
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser()
-    ap.add_argument("--model-throughput", default="gezavik", choices=["gezavik", "sigudra", "tukedra"])
+    ap.add_argument("--model-throughput", default="gezavik", choices=["gezavik", "sigudra", "tukedra", "purozen"])
     add_arguments(ap)
     return run(ap.parse_args(argv))
 

@@ -96,8 +96,9 @@ __global__ void post_norm_kernel(float* __restrict__ x, const TA* __restrict__ a
   }
 }
 
+// 0.5 z (1 + tanh(u)) with u = sqrt(2/pi) (z + 0.044715 z^3), written as z sigmoid(2u): one exponential
 __device__ __forceinline__ float mx_gelu_tanh(float z) {
-  return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+  return z * mx_sigmoid(1.5957691216057308f * (z + 0.044715f * z * z * z));
 }
 
 __device__ __forceinline__ float mx_act(float v, int act) {
@@ -120,6 +121,27 @@ __global__ void glu_act_kernel(const T* __restrict__ gate, long sg, const T* __r
     const float g = mx_act(s * ldf(gate + t * sg + c), act);
     stf(out + t * so + c, up != nullptr ? g * (s * ldf(up + t * su + c)) : g);
   }
+}
+
+// the same with 16-byte accesses: grid (rows, column chunks), V elements per thread; every row start and the
+// column count are multiples of V elements
+template <typename T, int V>
+__global__ void glu_act_vec_kernel(const T* __restrict__ gate, long sg, const T* __restrict__ up, long su,
+                                   const float* __restrict__ row_scale, int act, T* __restrict__ out, long so, int nv) {
+  typedef T vec __attribute__((ext_vector_type(V)));
+  const long t = blockIdx.x;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= nv) return;
+  const float s = row_scale != nullptr ? row_scale[t] : 1.0f;
+  const vec g = *reinterpret_cast<const vec*>(gate + t * sg + (long)c * V);
+  vec u, o;
+  if (up != nullptr) u = *reinterpret_cast<const vec*>(up + t * su + (long)c * V);
+#pragma unroll
+  for (int e = 0; e < V; ++e) {
+    const float a = mx_act(s * (float)g[e], act);
+    o[e] = (T)(up != nullptr ? a * (s * (float)u[e]) : a);
+  }
+  *reinterpret_cast<vec*>(out + t * so + (long)c * V) = o;
 }
 
 // one wave per token: the `top` largest scores (ties: the lower index) with the score as weight.
@@ -236,6 +258,20 @@ MX_API int mx_glu_act(const void* gate, long sg, const void* up, long su, const 
                       long so, int dt, int T, int n, hipStream_t st) {
   const long total = (long)T * n;
   if (total <= 0) return 0;
+  const int V = dt == 1 ? 4 : 8;                       // elements per 16 bytes
+  const bool aligned = n % V == 0 && sg % V == 0 && so % V == 0 && (up == nullptr || su % V == 0) &&
+                       ((size_t)gate | (size_t)out | (size_t)up) % 16 == 0 && (size_t)n / V <= 65535u * 256u;
+  if (aligned) {
+    const int nv = n / V;
+    dim3 grid(T, (nv + 255) / 256);
+    if (dt == 1)
+      glu_act_vec_kernel<float, 4><<<grid, 256, 0, st>>>((const float*)gate, sg, (const float*)up, su, row_scale, act,
+                                                         (float*)out, so, nv);
+    else
+      glu_act_vec_kernel<bf16, 8><<<grid, 256, 0, st>>>((const bf16*)gate, sg, (const bf16*)up, su, row_scale, act,
+                                                        (bf16*)out, so, nv);
+    MX_RETURN_LAUNCH();
+  }
   const int blocks = (int)((total + 255) / 256 < 16384 ? (total + 255) / 256 : 16384);
   MX_DISPATCH(dt, TT, glu_act_kernel<TT><<<blocks, 256, 0, st>>>((const TT*)gate, sg, (const TT*)up, su, row_scale, act,
                                                                   (TT*)out, so, n, total));

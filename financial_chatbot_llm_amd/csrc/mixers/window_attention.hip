@@ -60,8 +60,9 @@ __global__ void qk_norm_write_kernel(const T* __restrict__ q, long sq, const T* 
   sq2 = mx_block_sum(sq2, scratch);
   sk2 = mx_block_sum(sk2, scratch);
   const float cq = 1.0f / sqrtf(sq2 / (float)nq + eps), ck = 1.0f / sqrtf(sk2 / (float)nk + eps);
-  for (int i = threadIdx.x; i < nq; i += blockDim.x)
-    stf(qout + t * nq + i, qw != nullptr ? ldf(qr + i) * cq * qw[i] : ldf(qr + i));
+  if (qout != nullptr)       // null: the caller reads the projection's own q slice (no norm, no copy)
+    for (int i = threadIdx.x; i < nq; i += blockDim.x)
+      stf(qout + t * nq + i, qw != nullptr ? ldf(qr + i) * cq * qw[i] : ldf(qr + i));
   const int slot = slots[t];
   if (slot < 0) return;
   T* dst = cache + (long)slot * (nk + nv);
@@ -500,11 +501,13 @@ static bool wa_use_mfma() {
 }
 
 // q [T, nq], k [T, nk], v [T, nv] slices (row strides sq, sk, sv); qw [nq], kw [nk] f32 (null: no norm);
-// cache [pages*64, nk + nv]; qout [T, nq] contiguous; all of storage type dt
+// cache [pages*64, nk + nv]; qout [T, nq] contiguous, or null without a query norm (cache write only); all of
+// storage type dt
 MX_API int mx_qk_norm_write(const void* q, long sq, const void* k, long sk, const void* v, long sv, const float* qw,
                             const float* kw, float eps, const int* slots, void* cache, void* qout, int dt, int T,
                             int nq, int nk, int nv, hipStream_t st) {
   if (T <= 0) return 0;
+  if (qout == nullptr && qw != nullptr) return (int)hipErrorInvalidValue;
   MX_DISPATCH(dt, TT, qk_norm_write_kernel<TT><<<T, 256, 0, st>>>((const TT*)q, sq, (const TT*)k, sk, (const TT*)v, sv, qw,
                                                                   kw, eps, slots, (TT*)cache, (TT*)qout, nq, nk, nv));
   MX_RETURN_LAUNCH();

@@ -51,7 +51,7 @@ def example_config(width: int = 160, vocab: int = 768, pattern: str = "paAl", sc
         att = {"dim": 128, "heads": H, "kv_heads": G, "mask": {"keep_first": 4, "size": 1024},
                "rot": {"base": 10000.0, "dims": 64, "scaling": {"factor": 2.0}}, "scale": 1.0, "v_mix": True, "vdim": 128}
         lat = {"dim": 128, "heads": H, "kv_rank": 256, "scale": 128 ** -0.5, "vdim": 128}
-        dense = {"ff": 3 * width, "kind": "dense"}
+        dense = {"ff": 4 * width, "kind": "dense"}
     else:
         par = {"left": {"dim": 24, "heads": 6, "kv_heads": 2, "scale": 0.3, "vdim": 20}, "left_scale": 0.7,
                "right": {"width": 72}, "right_scale": 1.2}

@@ -717,22 +717,23 @@ def qk_norm_write(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, qw: Optiona
                   kw: Optional[torch.Tensor], eps: float, slots: torch.Tensor, cache: torch.Tensor) -> torch.Tensor:
     """Per token: RMS norm of the WHOLE query projection (all heads at once) times ``qw`` -> returned
     [T, nq]; the same for the key projection with ``kw``; the normed keys and the values go to cache
-    row ``slots[t]`` as [k | v] (< 0: no write).  ``qw``/``kw`` None: no norm."""
+    row ``slots[t]`` as [k | v] (< 0: no write).  ``qw``/``kw`` None: no norm (without ``qw`` the returned
+    queries are ``q`` itself, a column slice: nothing is copied)."""
     T, nq = q.shape
     nk, nv = k.shape[1], v.shape[1]
     assert cache.shape[-1] == nk + nv
     if N.use_native(q):
         assert q.dtype == k.dtype == v.dtype == cache.dtype
-        out = torch.empty((T, nq), dtype=q.dtype, device=q.device)
+        out = torch.empty((T, nq), dtype=q.dtype, device=q.device) if qw is not None else None
         N.mcall("mx_qk_norm_write", N.ptr(_rows(q)), q.stride(0), N.ptr(_rows(k)), k.stride(0), N.ptr(_rows(v)), v.stride(0),
                 N.ptr(qw), N.ptr(kw), float(eps), N.ptr(slots), N.ptr(cache), N.ptr(out), _dt(q), T, nq, nk, nv, N.stream())
-        return out
+        return out if out is not None else q
     rms = lambda t, w: (t.float() * torch.rsqrt(t.float().pow(2).mean(-1, keepdim=True) + eps) * w.float()  # noqa: E731
                         if w is not None else t.float())
     rows = torch.cat([rms(k, kw), v.float()], 1).to(cache.dtype)
     ok = slots >= 0
     cache.view(-1, nk + nv)[slots[ok].long()] = rows[ok]
-    return rms(q, qw).to(q.dtype)
+    return rms(q, qw).to(q.dtype) if qw is not None else q
 
 
 def window_attend(q: torch.Tensor, cache: torch.Tensor, cu: torch.Tensor, pos: torch.Tensor, bt: torch.Tensor,
