@@ -9,7 +9,10 @@ gated activations with a per-row scale and sigmoid top-k routing; and, for decod
 residual streams per token (hyper-connections), the fused stream update + read + RMS norm, a rotation
 of projected heads (two pair layouts, scaled frequencies, per-head RMS norm), matrix-state recurrences
 with one fixed decay per head, a chunked attention mask, top-k routing with a softmax over the chosen
-logits, and the logit scale / soft cap.
+logits, and the logit scale / soft cap; and, for pre-norm decoders with gated residual updates, a sigmoid
+gate and two weighted outputs on the fused residual update, attention with kept first tokens beyond a
+sliding window and with unnormalised sigmoid weights, a minimal gated recurrent unit, values blended
+across layers at the cache write, and linearly scaled rotation frequencies.
 
 Activations are bf16 or f32 (a model-wide choice); statistics, scores, softmax, recurrences and the
 residual stream are f32 either way.  CUDA(HIP) tensors run the kernels of ``libpenny_mixers.so``
