@@ -196,7 +196,7 @@ def test_other_sizes(device, dtype):
     """Sizes unlike the small default: odd head counts, key and value sizes that fill no wave and differ,
     a window longer than a page and one shorter than the kept first tokens, rotation over the whole head
     and over two entries, the first blending layer behind an attention layer that does not blend, three
-    blending layers, a large norm eps, other constants."""
+    blending layers, feed-forward widths of 1, 9 and 333, a large norm eps, other constants."""
     cfgd = small_config("alapaPaL", width=80, vocab=97)
     cfgd["norm"]["eps"] = 0.02
     L = cfgd["layers"]
@@ -214,6 +214,9 @@ def test_other_sizes(device, dtype):
     L[5]["mixer"]["right"].update(width=3)
     L[6]["mixer"].update(dim=16, vdim=8, heads=5, kv_heads=5, mask={"size": 64, "keep_first": 64}, scale=1.0)
     L[7]["mixer"].update(dim=70, vdim=5, heads=2, kv_rank=9, scale=0.2)
+    for l, ff in zip(L, (50, 9, 224, 1, 333, 0, 80, 0)):       # widths that are no multiple of the 16-byte accesses
+        if l["mlp"]:
+            l["mlp"]["ff"] = ff
     eng, sd = build(cfgd, device, dtype, blocks_=8)
     poison(eng)
     toks = tokens(150, cfgd["vocab"], 7)
