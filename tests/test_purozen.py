@@ -352,10 +352,10 @@ def test_batch_rows_do_not_depend_on_their_neighbours(device):
 # ---------------------------------------------------------------------------------------------------
 # window edges, kept first tokens, page borders, far keys: scores and states that stand out
 # ---------------------------------------------------------------------------------------------------
-def _paged(n, pages, width, g, table):
+def _paged(pages, width, table):
+    """An empty cache of ``pages`` pages and the row of position j under the page table."""
     row = lambda j: int(table[0, j // 64]) * 64 + j % 64  # noqa: E731
-    cache = torch.zeros(pages * 64, width)
-    return cache, row
+    return torch.zeros(pages * 64, width), row
 
 
 @pytest.mark.parametrize("device", DEVICES)
@@ -370,7 +370,7 @@ def test_window_and_kept_edges_stand_out(device, dtype, size, keep):
     H, G, D, P, pages, n = 6, 2, 16, 12, 4, 200
     g = torch.Generator().manual_seed(size)
     table = i32([[2, 0, 3, 1]])
-    cache, row = _paged(n, pages, G * (D + P), g, table)
+    cache, row = _paged(pages, G * (D + P), table)
     for j in range(n):
         cache[row(j), G * D:] = torch.randn(G * P, generator=g)           # values; keys stay zero
     chunks = [list(range(p0, p0 + 8)) for p0 in (size + keep, 60, 124, 188)]
